@@ -59,6 +59,13 @@ def _bezurax(path, dtype, device):
     return build_bezurax_from_dir(path, dtype=dtype, device=device)
 
 
+@register_model("Tilarax")
+def _tilarax(path, dtype, device):
+    from megatron_amd.models.tilarax import build_tilarax_from_dir
+
+    return build_tilarax_from_dir(path, dtype=dtype, device=device)
+
+
 @register_model("LlamaForCausalLM")
 def _llama(path, dtype, device):
     """HuggingFace Llama checkpoints -> GPTModel (single process, TP=1)."""

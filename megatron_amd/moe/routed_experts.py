@@ -1,4 +1,4 @@
-"""Routed clamped-GLU experts for the ragged serving path (single process, all
+"""Routed GLU experts for the ragged serving path (single process, all
 experts resident; the training-side MoE with token dispatchers is
 moe/moe_layer.py).
 
@@ -8,6 +8,9 @@ two largest scores; the selection rule of moe/router.py::group_limited_topk),
 weights = chosen scores / their sum * route_scale.
 Expert (no biases): g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit),
 y = g sigmoid(alpha g) (u + 1), output W_down y.
+Other designs choose by the raw logits and weigh by the softmax over the chosen
+logits (``score="softmax"``, optional router bias), and use the plain SiLU GLU
+y = g sigmoid(g) u (``activation="silu"``).
 Optional shared expert of the same form for every token, times
 sigmoid(w_sg . h); its gate row rides in the fp32 router GEMM.
 
@@ -36,8 +39,12 @@ from megatron_amd.ops import ragged as R
 class RoutedExpertsMLP(nn.Module):
     def __init__(self, hidden: int, experts: int, top: int, ff: int, limit: float, groups: int = 1,
                  keep: int = 1, route_scale: float = 1.0, shared_ff: Optional[int] = None,
-                 shared_limit: Optional[float] = None, alpha: float = 1.702, dtype=torch.bfloat16):
+                 shared_limit: Optional[float] = None, alpha: float = 1.702, score: str = "sigmoid",
+                 router_bias: bool = False, activation: str = "clamped", dtype=torch.bfloat16):
         super().__init__()
+        assert score in R.ROUTER_SCORES and activation in R.GLU_KINDS
+        assert score == "sigmoid" or groups <= 1, "group-limited choice is defined on sigmoid scores"
+        self.score, self.activation = score, activation
         assert top <= experts and experts % max(groups, 1) == 0
         if groups > 1:
             assert keep * (experts // groups) >= top, "the kept groups hold fewer experts than are chosen"
@@ -47,6 +54,8 @@ class RoutedExpertsMLP(nn.Module):
         self.shared_limit = float(shared_limit) if shared_ff else None
         # row ``experts`` (when there is a shared expert) is its gate vector
         self.w_router = nn.Parameter(torch.zeros(experts + (1 if shared_ff else 0), hidden, dtype=torch.float32))
+        self.b_router = (nn.Parameter(torch.zeros(experts + (1 if shared_ff else 0), dtype=torch.float32))
+                         if router_bias else None)
         self.w_gate_up = nn.Parameter(torch.zeros(experts, 2 * ff, hidden, dtype=dtype))   # [gate; up] per expert
         self.w_down = nn.Parameter(torch.zeros(experts, hidden, ff, dtype=dtype))
         if shared_ff:
@@ -55,7 +64,11 @@ class RoutedExpertsMLP(nn.Module):
 
     def route(self, h: torch.Tensor):
         """-> (ids [T, top], weights [T, top], the shared expert's gate logit [T, 1] or [T, 0])"""
-        return R.moe_router(h, self.w_router, self.experts, self.top, self.groups, self.keep, self.route_scale)
+        return R.moe_router(h, self.w_router, self.experts, self.top, self.groups, self.keep, self.route_scale,
+                            self.b_router, self.score)
+
+    def _glu(self, gu, limit, dtype):
+        return R.glu(gu, self.activation, limit, self.alpha, dtype)
 
     def _grouped_ok(self, h: torch.Tensor) -> bool:
         """bf16 on the GPU with 16-byte aligned rows: the grouped GEMM the training-side
@@ -70,12 +83,12 @@ class RoutedExpertsMLP(nn.Module):
         ids, weights, extra = self.route(h)
         shared = gate = None
         if self.shared_ff:
-            sy = R.clamped_glu(F.linear(h, self.ws_gate_up), self.shared_limit, self.alpha, h.dtype)
+            sy = self._glu(F.linear(h, self.ws_gate_up), self.shared_limit, h.dtype)
             shared = F.linear(sy, self.ws_down)
             gate = extra.reshape(-1)
         if R.expert_pairs_ok(h, K, self.ff):
             # few pairs (decoding): each pair streams its expert's matrices, no sort, no host read
-            down = R.expert_pairs(h, ids, self.w_gate_up, self.w_down, self.limit, self.alpha)
+            down = R.expert_pairs(h, ids, self.w_gate_up, self.w_down, self.limit, self.alpha, self.activation)
             inv = torch.arange(T * K, dtype=torch.int32, device=h.device).view(T, K)
             return R.moe_combine(down, inv, weights, shared, gate, add)
         flat = ids.reshape(-1).long()
@@ -87,7 +100,7 @@ class RoutedExpertsMLP(nn.Module):
             # one grouped GEMM per linear over the sorted pairs, group ends on the device: no host read
             offs = torch.cumsum(torch.bincount(flat, minlength=E), 0).to(torch.int32)
             gu = torch._grouped_mm(xs, self.w_gate_up.transpose(1, 2), offs=offs)
-            down = torch._grouped_mm(R.clamped_glu(gu, self.limit, self.alpha, h.dtype),
+            down = torch._grouped_mm(self._glu(gu, self.limit, h.dtype),
                                      self.w_down.transpose(1, 2), offs=offs)
         else:
             counts = torch.bincount(flat, minlength=E).tolist()   # the step's host read
@@ -96,6 +109,6 @@ class RoutedExpertsMLP(nn.Module):
             for e, n in enumerate(counts):
                 if n:
                     gu = F.linear(xs[at:at + n], self.w_gate_up[e])
-                    down[at:at + n] = F.linear(R.clamped_glu(gu, self.limit, self.alpha, h.dtype), self.w_down[e])
+                    down[at:at + n] = F.linear(self._glu(gu, self.limit, h.dtype), self.w_down[e])
                     at += n
         return R.moe_combine(down, inv.view(T, K).to(torch.int32), weights, shared, gate, add)

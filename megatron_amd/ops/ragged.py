@@ -8,6 +8,11 @@ softmax sink, xIELU.
 grouped RMS norm, whole-projection q/k norm with cache store, pooled-block
 completion and attention over a sliding window plus pooled blocks, generalized
 delta rule, expert routing, clamped GLU, pair-streaming experts, expert combine.
+``_talking_ops``: post-sublayer norm with a depth-weighted residual history,
+per-head q/k norm with pairwise rotation, value mixing and cache store, chunked
+talking-heads attention, tanh-GELU; it also carries the embedding, mLSTM and
+routed-expert kernels of the other two (same sources), so that a model built
+on it compiles nothing else.
 
 Dispatch rule (same as megatron_amd.ops): tensors on a HIP device run the
 CDNA4 kernels of the extension (csrc/ragged/*.hip, csrc/hybrid/*.hip) and RAISE
@@ -28,17 +33,18 @@ from megatron_amd.ops.ragged_reference import rope_table  # noqa: F401  (host-si
 
 _C = None      # _ragged_ops: latent attention, mLSTM, minGRU, hyper-connections, canon conv, xIELU
 _H = None      # _hybrid_ops: grouped norm, pooled-window attention, delta rule, routed experts
+_K = None      # _talking_ops: post-norm with depth history, talking-heads attention (+ shared kernels)
 _IMPORT_ERROR: Optional[str] = None
 _IMPORT_ERRORS = {}
 
 # setup.py extension key -> module name; a model names the keys it needs in
 # ``native_extensions`` and a serving process builds only those on first use
-EXTENSIONS = {"ragged": "_ragged_ops", "hybrid": "_hybrid_ops"}
+EXTENSIONS = {"ragged": "_ragged_ops", "hybrid": "_hybrid_ops", "talking": "_talking_ops"}
 
 
 def _load(key: str = "ragged"):
-    global _C, _H, _IMPORT_ERROR
-    cur = _C if key == "ragged" else _H
+    global _C, _H, _K, _IMPORT_ERROR
+    cur = {"ragged": _C, "hybrid": _H, "talking": _K}[key]
     if cur is not None:
         return cur
     try:
@@ -47,8 +53,10 @@ def _load(key: str = "ragged"):
         mod = importlib.import_module("megatron_amd.ops." + EXTENSIONS[key])  # built in-tree (setup.py)
         if key == "ragged":
             _C = mod
-        else:
+        elif key == "hybrid":
             _H = mod
+        else:
+            _K = mod
         return mod
     except Exception as e:  # noqa: BLE001
         _IMPORT_ERRORS[key] = repr(e)
@@ -59,6 +67,7 @@ def _load(key: str = "ragged"):
 
 _load("ragged")
 _load("hybrid")
+_load("talking")
 
 
 def build_extension(key: str, verbose: bool = False) -> None:
@@ -114,6 +123,21 @@ def _native_h(x: torch.Tensor) -> bool:
     return True
 
 
+def _pick(x: torch.Tensor, *keys):
+    """The first built extension among ``keys`` for a GPU tensor (several
+    extensions carry the same kernel), None for the torch path; raises when a
+    GPU tensor finds none of them."""
+    if not x.is_cuda or os.environ.get("MEGATRON_AMD_FORCE_REFERENCE", "0") == "1":
+        return None
+    for key in keys:
+        mod = {"ragged": _C, "hybrid": _H, "talking": _K}[key]
+        if mod is not None:
+            return mod
+    raise RuntimeError(
+        f"none of the HIP extensions {keys} is built but a GPU tensor hit the ops layer "
+        f"(import errors: {_IMPORT_ERRORS}). Run megatron_amd.ops.ragged.build_extension('{keys[0]}').")
+
+
 _EMPTY = {}
 
 
@@ -161,8 +185,9 @@ def mingru_scan(zxg, bias_z, bias_x, state, batch, out_dtype):
 
 def mlstm_scan(qkvg, gates, bias_i, bias_f, norm_w, heads, dim, vdim, cap, eps,
                state_S, state_n, state_m, batch, out_dtype):
-    if _native(qkvg):
-        return _C.mlstm_scan(qkvg, gates, bias_i, bias_f, norm_w, heads, dim, vdim, float(cap), float(eps),
+    ext = _pick(qkvg, "ragged", "talking")
+    if ext is not None:
+        return ext.mlstm_scan(qkvg, gates, bias_i, bias_f, norm_w, heads, dim, vdim, float(cap), float(eps),
                              state_S, state_n, state_m, batch.cu_tokens, batch.slots)
     return ref.mlstm_scan(qkvg, gates, bias_i, bias_f, norm_w, heads, dim, vdim, cap, eps,
                           state_S, state_n, state_m, batch, out_dtype)
@@ -232,16 +257,18 @@ def gate_heads(x, gate_pre, heads):
 
 
 def embed_plain(tokens, embed):
-    if _native_h(embed):
-        return _H.embed_plain(tokens, embed)
+    ext = _pick(embed, "hybrid", "talking")
+    if ext is not None:
+        return ext.embed_plain(tokens, embed)
     return ref.embed_plain(tokens, embed)
 
 
 def residual_group_norm(x, y, w_a, w_b, groups, eps, out_dtype):
     """x fp32 [T, W] += y in place (y may be None); -> (norm(x) w_a, norm(x) w_b or None)."""
-    if _native_h(x):
+    ext = _pick(x, "hybrid", "talking")
+    if ext is not None:
         d = x.device
-        h_a, h_b = _H.residual_group_norm(x, y if y is not None else _none(d), w_a,
+        h_a, h_b = ext.residual_group_norm(x, y if y is not None else _none(d), w_a,
                                           w_b if w_b is not None else _none(d), int(groups), float(eps),
                                           out_dtype == torch.bfloat16)
         return h_a, (h_b if w_b is not None else None)
@@ -304,18 +331,31 @@ def moe_route(logits, experts, top, groups, keep, scale):
     return ref.moe_route(logits, experts, top, groups, keep, scale)
 
 
+GLU_KINDS = {"clamped": 0, "silu": 1}
+
+
 def clamped_glu(gu, limit, alpha, out_dtype):
-    if _native_h(gu):
-        return _H.clamped_glu(gu, float(limit), float(alpha))
+    return glu(gu, "clamped", limit, alpha, out_dtype)
+
+
+def glu(gu, act, limit, alpha, out_dtype):
+    """gu [N, 2F] = [gate | up] -> [N, F]: "clamped": min(g, limit) sigmoid(alpha g) (clamp(u) + 1);
+    "silu": g sigmoid(g) u."""
+    ext = _pick(gu, "hybrid", "talking")
+    if ext is not None:
+        return ext.clamped_glu(gu, float(limit), float(alpha), GLU_KINDS[act])
+    if act == "silu":
+        return ref.silu_glu(gu, out_dtype)
     return ref.clamped_glu(gu, limit, alpha, out_dtype)
 
 
 def moe_combine(down, inv, weights, shared, shared_gate, add):
-    if _native_h(down):
+    ext = _pick(down, "hybrid", "talking")
+    if ext is not None:
         d = down.device
-        return _H.moe_combine(down, inv, weights, shared if shared is not None else _none(d),
-                              shared_gate if shared is not None else _none(d),
-                              add if add is not None else _none(d))
+        return ext.moe_combine(down, inv, weights, shared if shared is not None else _none(d),
+                               shared_gate if shared is not None else _none(d),
+                               add if add is not None else _none(d))
     return ref.moe_combine(down, inv, weights, shared, shared_gate, add)
 
 
@@ -324,19 +364,89 @@ PAIR_PATH_MAX = 32      # (token, choice) pairs up to which every pair streams i
 
 def expert_pairs_ok(h, top, ff) -> bool:
     """Steps with few pairs (decoding) skip the sort by expert: see csrc/hybrid/experts.hip."""
-    return (h.is_cuda and _H is not None and os.environ.get("MEGATRON_AMD_FORCE_REFERENCE", "0") != "1"
+    return (h.is_cuda and (_H is not None or _K is not None)
+            and os.environ.get("MEGATRON_AMD_FORCE_REFERENCE", "0") != "1"
             and h.shape[0] * top <= PAIR_PATH_MAX and h.shape[1] % 8 == 0 and ff % 8 == 0
             and max(h.shape[1], ff) <= 15360)
 
 
-def expert_pairs(h, ids, w_gate_up, w_down, limit, alpha):
-    if _native_h(h):
-        return _H.expert_pairs(h, ids, w_gate_up, w_down, float(limit), float(alpha))
-    return ref.expert_pairs(h, ids, w_gate_up, w_down, limit, alpha)
+def expert_pairs(h, ids, w_gate_up, w_down, limit, alpha, act="clamped"):
+    ext = _pick(h, "hybrid", "talking")
+    if ext is not None:
+        return ext.expert_pairs(h, ids, w_gate_up, w_down, float(limit), float(alpha), GLU_KINDS[act])
+    return ref.expert_pairs(h, ids, w_gate_up, w_down, limit, alpha, act)
 
 
-def moe_router(h, w_router, experts, top, groups, keep, scale):
-    """-> (ids [T, top] int32, weights [T, top] fp32, raw logits of the rows beyond the experts)"""
-    if _native_h(h) and h.shape[1] <= 15360 and w_router.shape[0] <= 512:
-        return _H.moe_router(h, w_router, int(experts), int(top), int(groups), int(keep), float(scale))
-    return ref.moe_router(h, w_router, experts, top, groups, keep, scale)
+ROUTER_SCORES = {"sigmoid": 0, "softmax": 1}
+
+
+def moe_router(h, w_router, experts, top, groups, keep, scale, bias=None, score="sigmoid"):
+    """-> (ids [T, top] int32, weights [T, top] fp32, raw logits of the rows beyond the experts)
+
+    score "sigmoid": sigmoid scores, group-limited choice, weights = chosen scores / their sum * scale;
+    score "softmax": the largest logits are chosen, weights = softmax over the chosen logits."""
+    ext = _pick(h, "hybrid", "talking")
+    if ext is not None and h.shape[1] <= 15360 and w_router.shape[0] <= 512:
+        return ext.moe_router(h, w_router, bias if bias is not None else _none(h.device), int(experts), int(top),
+                              int(groups), int(keep), float(scale), ROUTER_SCORES[score])
+    return ref.moe_router(h, w_router, experts, top, groups, keep, scale, bias, score)
+
+
+# ---------------------------------------------------------------------------
+# ops of the talking extension: post-sublayer norm with a depth-weighted
+# residual history, per-head q/k norm with pairwise rotation and value mixing,
+# chunked talking-heads attention, tanh-GELU
+# ---------------------------------------------------------------------------
+
+pair_freqs = ref.pair_freqs
+
+
+def _native_k(x: torch.Tensor) -> bool:
+    return _pick(x, "talking") is not None
+
+
+def post_norm_add(x, y, w, eps, out_dtype, hist=None, depth=0, dwa=None):
+    """x fp32 [T, W] <- x + rms(y) (1 + w) in place (y may be None); with ``hist``:
+    hist[depth] <- x, x <- sum_{j <= depth} dwa[j] hist[j].  -> x in out_dtype."""
+    if _native_k(x):
+        d = x.device
+        return _K.post_norm_add(x, y if y is not None else _none(d), w if y is not None else _none(d), float(eps),
+                                out_dtype == torch.bfloat16, hist if hist is not None else _none(d), int(depth),
+                                dwa if hist is not None else _none(d))
+    return ref.post_norm_add(x, y, w, eps, out_dtype, hist, depth, dwa)
+
+
+def head_norm_rope_store(proj, heads, kv_heads, dim, vdim, q_norm, k_norm, eps, freqs, v_first, lam, pool, batch):
+    if _native_k(proj):
+        d = proj.device
+        return _K.head_norm_rope_store(proj, int(heads), int(kv_heads), int(dim), int(vdim), q_norm, k_norm,
+                                       float(eps), freqs, v_first if v_first is not None else _none(d),
+                                       lam if v_first is not None else _none(d), pool, batch.tok_pos, batch.tok_row)
+    return ref.head_norm_rope_store(proj, heads, kv_heads, dim, vdim, q_norm, k_norm, eps, freqs, v_first, lam,
+                                    pool, batch)
+
+
+def talking_attention(q, pool, heads, kv_heads, dim, vdim, scale, temp, talk, chunk, batch, out_dtype):
+    """-> [T, heads * vdim] in out_dtype"""
+    if _native_k(q):
+        if (q.dtype == torch.bfloat16 and dim % 8 == 0 and vdim % 8 == 0 and dim <= 256 and vdim <= 256
+                and os.environ.get("MEGATRON_AMD_NO_MFMA_TALKING", "0") != "1"):
+            # matrix-core kernel: 64 (token, head-in-group) rows per workgroup and (key head, value
+            # head) pair; steps with few rows (decode) also split the key tiles over workgroups
+            tiles = batch.row_tiles(heads // kv_heads, q.device)
+            nblk = tiles.shape[0] * kv_heads * kv_heads
+            keys = min(batch.max_context, chunk) if chunk > 0 else batch.max_context
+            nsplit = max(1, min((keys + 63) // 64, 1024 // max(nblk, 1), 64))
+            return _K.talking_attention_mfma(q, pool, int(heads), int(kv_heads), int(dim), int(vdim), float(scale),
+                                             temp, talk, int(chunk), tiles, batch.cu_tokens, batch.start_pos,
+                                             batch.block_tables, int(batch.block_size), int(nsplit))
+        return _K.talking_attention(q, pool, int(heads), int(kv_heads), int(dim), int(vdim), float(scale), temp,
+                                    talk, int(chunk), batch.tok_req, batch.tok_pos, batch.block_tables,
+                                    int(batch.block_size))
+    return ref.talking_attention(q, pool, heads, kv_heads, dim, vdim, scale, temp, talk, chunk, batch, out_dtype)
+
+
+def gelu_tanh(z, out_dtype):
+    if _native_k(z):
+        return _K.gelu_tanh(z)
+    return ref.gelu_tanh(z, out_dtype)

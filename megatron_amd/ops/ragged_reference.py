@@ -403,22 +403,150 @@ def moe_combine(down, inv, weights, shared, shared_gate, add):
     return y
 
 
-def expert_pairs(h, ids, w_gate_up, w_down, limit, alpha):
+def expert_pairs(h, ids, w_gate_up, w_down, limit, alpha, act="clamped"):
     """Every (token, choice) pair through its expert, rows in pair order
-    (token-major): clamped GLU of [gate; up] x, then the down product."""
+    (token-major): GLU of [gate; up] x (clamped or SiLU), then the down product."""
     T, K = ids.shape
     out = torch.empty(T * K, h.shape[1], dtype=h.dtype, device=h.device)
     for t in range(T):
         for k in range(K):
             e = int(ids[t, k])
-            y = clamped_glu(F.linear(h[t:t + 1], w_gate_up[e]), limit, alpha, h.dtype)
+            gu = F.linear(h[t:t + 1], w_gate_up[e])
+            y = silu_glu(gu, h.dtype) if act == "silu" else clamped_glu(gu, limit, alpha, h.dtype)
             out[t * K + k] = F.linear(y, w_down[e])[0]
     return out
 
 
-def moe_router(h, w_router, experts, top, groups, keep, scale):
-    """Router in one call: fp32 logits of all rows of w_router (the rows beyond
-    ``experts`` are returned raw), then moe_route.  -> (ids, weights, extra [T, rows - experts])"""
-    logits = F.linear(h.float(), w_router.float())
-    ids, weights = moe_route(logits, experts, top, groups, keep, scale)
+def moe_router(h, w_router, experts, top, groups, keep, scale, bias=None, score="sigmoid"):
+    """Router in one call: fp32 logits of all rows of w_router (+ bias; the rows
+    beyond ``experts`` are returned raw), then moe_route (score "sigmoid") or
+    moe_route_softmax (score "softmax").  -> (ids, weights, extra [T, rows - experts])"""
+    logits = F.linear(h.float(), w_router.float(), bias.float() if bias is not None else None)
+    if score == "softmax":
+        ids, weights = moe_route_softmax(logits[:, :experts], top)
+    else:
+        ids, weights = moe_route(logits, experts, top, groups, keep, scale)
     return ids, weights, logits[:, experts:].contiguous()
+
+
+# ---------------------------------------------------------------------------
+# post-sublayer norm with depth-weighted residual history, per-head q/k norm
+# with pairwise rotation and value mixing, chunked talking-heads attention,
+# tanh-GELU, routing by softmax over the chosen logits, SiLU GLU
+# ---------------------------------------------------------------------------
+
+
+def post_norm_add(x, y, w, eps, out_dtype, hist, depth, dwa):
+    """x fp32 [T, W] <- x + y / sqrt(mean(y^2) + eps) * (1 + w) in place (skipped
+    when ``y`` is None).  With ``hist`` ([layers + 1, T, W] fp32, entry 0 = the
+    embedding output): hist[depth] <- x, then x <- sum_{j <= depth} dwa[j] hist[j].
+    Returns x in ``out_dtype`` (the next sublayer's GEMM input)."""
+    if y is not None:
+        yf = y.float()
+        x.add_(yf * torch.rsqrt((yf * yf).mean(-1, keepdim=True) + eps) * (1.0 + w.float()))
+    if hist is not None:
+        hist[depth].copy_(x)
+        x.copy_(torch.einsum("j,jtw->tw", dwa.float()[:depth + 1], hist[:depth + 1]))
+    return x if out_dtype == torch.float32 else x.to(out_dtype)
+
+
+def pair_freqs(dims, base, device=None):
+    """f_i = base^(-2i/dims), i < dims/2, rounded once to fp32."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims).to(torch.float32).to(device)
+
+
+def _rotate_pairs(x, pos, freqs):
+    """x [T, heads, d] fp32: entries (2i, 2i+1), i < len(freqs), rotated by pos * f_i."""
+    n = freqs.numel()
+    if n == 0:
+        return x
+    ang = pos.float()[:, None, None] * freqs.float()[None, None, :]
+    c, s = torch.cos(ang), torch.sin(ang)
+    u, v = x[..., 0:2 * n:2], x[..., 1:2 * n:2]
+    out = x.clone()
+    out[..., 0:2 * n:2] = u * c - v * s
+    out[..., 1:2 * n:2] = v * c + u * s
+    return out
+
+
+def head_norm_rope_store(proj, heads, kv_heads, dim, vdim, q_norm, k_norm, eps, freqs, v_first, lam, pool, batch):
+    """proj [T, H*dim | G*dim | G*vdim] = [q | k | v] of the step's tokens.
+    Every head of q and k is divided by its own root mean square and scaled by a
+    weight [dim] that all heads share, then its first 2 * len(freqs) entries are
+    rotated in neighbouring pairs by the token's position.  With ``v_first``
+    ([T, G*vdim], another layer's values of the same tokens):
+    v <- (1 - lam) v + lam v_first.  Cache row <- [k | v]; returns q [T, H*dim]."""
+    T = proj.shape[0]
+    H, G, D, V = heads, kv_heads, dim, vdim
+    pf = proj.float()
+    q = pf[:, :H * D].view(T, H, D)
+    k = pf[:, H * D:(H + G) * D].view(T, G, D)
+    v = pf[:, (H + G) * D:(H + G) * D + G * V]
+    q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + eps) * q_norm.float()
+    k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + eps) * k_norm.float()
+    q = _rotate_pairs(q, batch.tok_pos, freqs)
+    k = _rotate_pairs(k, batch.tok_pos, freqs)
+    if v_first is not None:
+        lf = lam.float().reshape(())
+        v = (1.0 - lf) * v + lf * v_first.float()
+    pool[batch.tok_row] = torch.cat([k.reshape(T, G * D), v], dim=-1).to(pool.dtype)
+    return q.reshape(T, H * D).to(proj.dtype)
+
+
+def talking_attention(q, pool, heads, kv_heads, dim, vdim, scale, temp, talk, chunk, batch, out_dtype):
+    """Softmax attention over the paged cache (rows [G*dim keys | G*vdim values])
+    whose weights are mixed over the heads after the softmax:
+        s_g(i, j) = q_g(i) . k_kv(g)(j) * scale * temp[g],   P_g = softmax_j s_g
+        o_h(i) = sum_j (sum_g talk[h, g] P_g(i, j)) v_kv(h)(j)
+    Position i sees j <= i with floor(j / chunk) = floor(i / chunk) (chunk <= 0:
+    every j <= i).  -> [T, H*vdim]."""
+    T = q.shape[0]
+    H, G, D, V = heads, kv_heads, dim, vdim
+    rep = H // G
+    bs = batch.block_size
+    dev = q.device
+    out = torch.empty(T, H * V, dtype=out_dtype, device=dev)
+    kvh = torch.arange(H, device=dev) // rep
+    for r, a, b, start, slot in _spans(batch):
+        n = b - a
+        L = start + n
+        lo = (start // chunk) * chunk if chunk > 0 else 0          # nothing older is visible to this step
+        table = torch.as_tensor(batch.host_tables[r], dtype=torch.long, device=dev)
+        kv = pool[_rows_of(table, L, bs, dev)[lo:]].float()
+        keys = kv[:, :G * D].view(-1, G, D)
+        vals = kv[:, G * D:].view(-1, G, V)
+        qi = torch.arange(start, L, device=dev)
+        j = torch.arange(lo, L, device=dev)
+        ok = j[None, :] <= qi[:, None]
+        if chunk > 0:
+            ok = ok & (torch.div(j, chunk, rounding_mode="floor")[None, :]
+                       == torch.div(qi, chunk, rounding_mode="floor")[:, None])
+        qq = q[a:b].float().view(n, H, D)
+        s = torch.einsum("nhd,lhd->nhl", qq, keys[:, kvh]) * (scale * temp.float())[None, :, None]
+        s = s.masked_fill(~ok[:, None, :], float("-inf"))
+        p = torch.softmax(s, dim=-1)
+        pm = torch.einsum("hg,ngl->nhl", talk.float(), p)
+        o = torch.einsum("nhl,lhv->nhv", pm, vals[:, kvh])
+        out[a:b] = o.reshape(n, H * V).to(out_dtype)
+    return out
+
+
+def gelu_tanh(z, out_dtype):
+    """0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))"""
+    zf = z.float()
+    return (0.5 * zf * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (zf + 0.044715 * zf * zf * zf)))).to(out_dtype)
+
+
+def silu_glu(gu, out_dtype):
+    """gu [N, 2F] = [gate | up]: y = gate sigmoid(gate) up."""
+    F_ = gu.shape[1] // 2
+    g, u = gu[:, :F_].float(), gu[:, F_:].float()
+    return (g * torch.sigmoid(g) * u).to(out_dtype)
+
+
+def moe_route_softmax(logits, top):
+    """The ``top`` largest logits are chosen; weights = softmax over the chosen
+    logits only.  -> (ids [T, top] int32, weights [T, top] fp32)."""
+    val, idx = logits.float().topk(top, dim=-1)
+    return idx.to(torch.int32), torch.softmax(val, dim=-1)

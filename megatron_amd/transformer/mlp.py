@@ -74,3 +74,20 @@ class XieluMLP(nn.Module):
         from megatron_amd.ops import ragged as R
 
         return F.linear(R.xielu(F.linear(h, self.w_up), self.act, h.dtype), self.w_down)
+
+
+class GeluMLP(nn.Module):
+    """Dense two-matrix feed-forward without biases, activation = the tanh form
+    of GELU (ops.ragged.gelu_tanh).  Plain replicated weights (serving path)."""
+
+    def __init__(self, hidden: int, ffn: int, dtype=torch.bfloat16):
+        super().__init__()
+        self.w_up = nn.Parameter(torch.zeros(ffn, hidden, dtype=dtype))
+        self.w_down = nn.Parameter(torch.zeros(hidden, ffn, dtype=dtype))
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        import torch.nn.functional as F
+
+        from megatron_amd.ops import ragged as R
+
+        return F.linear(R.gelu_tanh(F.linear(h, self.w_up), h.dtype), self.w_down)
