@@ -201,7 +201,7 @@ def load_tilarax_state(model: TilaraxModel, tensors: Dict[str, torch.Tensor]) ->
                 mx.k_norm.data.copy_(get(a + "k.norm"))
                 mx.temp.data.copy_(get(a + "temp"))
                 mx.talk.data.copy_(get(a + "talk"))
-                if mx.value_mix and a + "vmix" in tensors:      # the first mixing layer never reads its own
+                if a + "vmix" in tensors:                       # the first mixing layer never reads its own
                     mx.lam.data.copy_(get(a + "vmix").reshape(1))
                 mx.w_out.data.copy_(get(a + "o"))
                 mx.b_out.data.copy_(get(a + "o.b"))

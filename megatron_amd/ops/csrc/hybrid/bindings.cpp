@@ -9,13 +9,13 @@ std::vector<torch::Tensor> residual_group_norm(torch::Tensor x, torch::Tensor y,
                                                int64_t groups, double eps, bool out_bf16);
 std::vector<torch::Tensor> moe_route(torch::Tensor logits, int64_t E, int64_t top, int64_t groups, int64_t keep,
                                      double scale);
-std::vector<torch::Tensor> moe_router(torch::Tensor h, torch::Tensor wr, int64_t E, int64_t top, int64_t groups,
-                                      int64_t keep, double scale);
-torch::Tensor clamped_glu(torch::Tensor gu, double limit, double alpha);
+std::vector<torch::Tensor> moe_router(torch::Tensor h, torch::Tensor wr, torch::Tensor bias, int64_t E, int64_t top,
+                                      int64_t groups, int64_t keep, double scale, int64_t score);
+torch::Tensor clamped_glu(torch::Tensor gu, double limit, double alpha, int64_t kind);
 torch::Tensor moe_combine(torch::Tensor down, torch::Tensor inv, torch::Tensor wts, torch::Tensor shared,
                           torch::Tensor gate, torch::Tensor add);
 torch::Tensor expert_pairs(torch::Tensor h, torch::Tensor ids, torch::Tensor wgu, torch::Tensor wd, double limit,
-                           double alpha);
+                           double alpha, int64_t kind);
 torch::Tensor qk_norm_store(torch::Tensor proj, int64_t q_off, int64_t qw, int64_t k_off, int64_t kw, int64_t v_off,
                             int64_t vw, torch::Tensor wq, torch::Tensor wk, double eps, torch::Tensor pool,
                             torch::Tensor tok_row);

@@ -1,4 +1,4 @@
-// Routed clamped-GLU experts for steps with few (token, choice) pairs
+// Routed GLU experts (clamped, kind 0, or SiLU, kind 1) for steps with few (token, choice) pairs
 // (decoding): every pair reads its expert's matrices directly, no sorting, no
 // host read.  Two kernels:
 //   y[pair, f]   = act(W_gate[e][f] . x, W_up[e][f] . x)     grid (pair, tiles of rows f)
@@ -28,7 +28,7 @@ __device__ __forceinline__ void load8<float>(const float* p, float* v) {
 template <typename T>
 __global__ __launch_bounds__(256) void expert_gate_up_kernel(
     const T* __restrict__ h, const int* __restrict__ ids, const T* __restrict__ wgu, T* __restrict__ y, int K,
-    int W, int F, float limit, float alpha) {
+    int W, int F, float limit, float alpha, int kind) {
   extern __shared__ float xs[];                  // the token's input, fp32
   const int pair = blockIdx.x, t = pair / K;
   const long e = ids[pair];
@@ -58,9 +58,13 @@ __global__ __launch_bounds__(256) void expert_gate_up_kernel(
       // the products' results take the storage type's rounding, as a GEMM's output would
       float g = ag, u = au;
       if (sizeof(T) == 2) { g = sbf2f(f2sbf(g)); u = sbf2f(f2sbf(u)); }
-      g = fminf(g, limit);
-      u = fminf(fmaxf(u, -limit), limit);
-      stf(y + (long)pair * F + f, g * sigmoidf_(alpha * g) * (u + 1.f));
+      if (kind == 0) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        stf(y + (long)pair * F + f, g * sigmoidf_(alpha * g) * (u + 1.f));
+      } else {
+        stf(y + (long)pair * F + f, g * sigmoidf_(g) * u);
+      }
     }
   }
 }
@@ -94,7 +98,8 @@ __global__ __launch_bounds__(256) void expert_down_kernel(const T* __restrict__ 
 
 // h [T, W], ids [T, K] -> rows [T * K, W] in pair order (token-major)
 torch::Tensor expert_pairs(torch::Tensor h, torch::Tensor ids, torch::Tensor wgu, torch::Tensor wd, double limit,
-                           double alpha) {
+                           double alpha, int64_t kind) {
+  TORCH_CHECK(kind == 0 || kind == 1, "GLU kind: 0 clamped, 1 SiLU");
   TORCH_CHECK(h.is_cuda() && h.dim() == 2 && h.is_contiguous());
   check_i32(ids, "ids");
   TORCH_CHECK(wgu.is_contiguous() && wgu.dim() == 3 && wd.is_contiguous() && wd.dim() == 3);
@@ -113,7 +118,7 @@ torch::Tensor expert_pairs(torch::Tensor h, torch::Tensor ids, torch::Tensor wgu
   RAGGED_DISPATCH(h, {
     hipLaunchKernelGGL((expert_gate_up_kernel<T>), dim3(N, (F + EP_ROWS - 1) / EP_ROWS), dim3(256),
         (size_t)W * sizeof(float), stream, (const T*)h.data_ptr(), ids.data_ptr<int>(), (const T*)wgu.data_ptr(),
-        (T*)y.data_ptr(), K, W, F, (float)limit, (float)alpha);
+        (T*)y.data_ptr(), K, W, F, (float)limit, (float)alpha, (int)kind);
     hipLaunchKernelGGL((expert_down_kernel<T>), dim3(N, (W + EP_ROWS - 1) / EP_ROWS), dim3(256),
         (size_t)F * sizeof(float), stream, (const T*)y.data_ptr(), ids.data_ptr<int>(), (const T*)wd.data_ptr(),
         (T*)out.data_ptr(), W, F);

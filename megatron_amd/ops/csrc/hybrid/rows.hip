@@ -177,8 +177,10 @@ std::vector<torch::Tensor> moe_route(torch::Tensor logits, int64_t E, int64_t to
 }
 
 // ---------------------------------------------------------------------------
-// router in one kernel: logits = W_r h in fp32 (W_r fp32, h from its storage
-// type), sigmoid scores, group-limited top-k, weights; rows beyond the experts
+// router in one kernel: logits = W_r h (+ bias) in fp32 (W_r fp32, h from its
+// storage type), then either sigmoid scores, group-limited top-k and weights =
+// chosen scores / their sum * scale (score 0), or the largest logits and
+// weights = softmax over the chosen logits (score 1); rows beyond the experts
 // (a shared expert's gate vector) are returned as raw logits.
 // One workgroup per token: its eight waves take the rows of W_r in turn (16 B
 // loads, four partial sums), one thread selects from the scores in LDS.
@@ -189,8 +191,9 @@ constexpr int RF_THREADS = 512;
 
 template <typename T>
 __global__ __launch_bounds__(RF_THREADS) void moe_router_kernel(
-    const T* __restrict__ h, const float* __restrict__ wr, int W, int rows, int E, int top, int groups, int keep,
-    float scale, int* __restrict__ ids, float* __restrict__ wts, float* __restrict__ extra) {
+    const T* __restrict__ h, const float* __restrict__ wr, const float* __restrict__ bias, int W, int rows, int E,
+    int top, int groups, int keep, float scale, int score, int* __restrict__ ids, float* __restrict__ wts,
+    float* __restrict__ extra) {
   extern __shared__ __align__(16) float xs[];    // the token's input, fp32
   __shared__ float sc[RF_MAX_ROWS];
   const long t = blockIdx.x;
@@ -208,9 +211,10 @@ __global__ __launch_bounds__(RF_THREADS) void moe_router_kernel(
       a0 += w[0] * x[0]; a1 += w[1] * x[1]; a2 += w[2] * x[2]; a3 += w[3] * x[3];
     }
     for (int d = W4 + lane; d < W; d += WAVE) a0 += row[d] * xs[d];
-    const float a = wave_reduce_sum((a0 + a1) + (a2 + a3));
+    float a = wave_reduce_sum((a0 + a1) + (a2 + a3));
     if (lane == 0) {
-      if (e < E) sc[e] = sigmoidf_(a);
+      if (bias != nullptr) a += bias[e];
+      if (e < E) sc[e] = score == 0 ? sigmoidf_(a) : a;
       else extra[t * (rows - E) + (e - E)] = a;
     }
   }
@@ -251,8 +255,21 @@ __global__ __launch_bounds__(RF_THREADS) void moe_router_kernel(
     }
     chosen[n] = best < 0 ? 0 : best;
     cs[n] = best < 0 ? 0.f : bv;
-    if (best >= 0) sc[best] = -2.f;               // taken
+    if (best >= 0) sc[best] = -INFINITY;          // taken
     sum += cs[n];
+  }
+  if (score != 0) {                               // softmax over the chosen logits; cs[0] is the largest
+    sum = 0.f;
+    const float top0 = cs[0];
+    for (int n = 0; n < top; ++n) {
+      cs[n] = expf(cs[n] - top0);
+      sum += cs[n];
+    }
+    for (int n = 0; n < top; ++n) {
+      ids[t * top + n] = chosen[n];
+      wts[t * top + n] = cs[n] / sum;
+    }
+    return;
   }
   for (int n = 0; n < top; ++n) {
     ids[t * top + n] = chosen[n];
@@ -260,10 +277,16 @@ __global__ __launch_bounds__(RF_THREADS) void moe_router_kernel(
   }
 }
 
-std::vector<torch::Tensor> moe_router(torch::Tensor h, torch::Tensor wr, int64_t E, int64_t top, int64_t groups,
-                                      int64_t keep, double scale) {
+std::vector<torch::Tensor> moe_router(torch::Tensor h, torch::Tensor wr, torch::Tensor bias, int64_t E, int64_t top,
+                                      int64_t groups, int64_t keep, double scale, int64_t score) {
   TORCH_CHECK(h.is_cuda() && h.dim() == 2 && h.is_contiguous());
   check_f32(wr, "router weight");
+  const bool has_bias = bias.numel() > 0;
+  if (has_bias) {
+    check_f32(bias, "router bias");
+    TORCH_CHECK(bias.numel() == wr.size(0), "one bias per router row");
+  }
+  TORCH_CHECK(score == 0 || (score == 1 && groups == 1), "score: 0 sigmoid (groups allowed), 1 softmax over the chosen");
   const int T_ = h.size(0), W = h.size(1), rows = wr.size(0);
   TORCH_CHECK(wr.dim() == 2 && wr.size(1) == W && E >= 1 && E <= rows && rows <= RF_MAX_ROWS);
   TORCH_CHECK(top >= 1 && top <= RT_MAX_TOP && top <= E, "experts chosen per token");
@@ -276,28 +299,36 @@ std::vector<torch::Tensor> moe_router(torch::Tensor h, torch::Tensor wr, int64_t
   if (T_ == 0) return {ids, wts, extra};
   auto stream = at::cuda::getCurrentHIPStream();
   RAGGED_DISPATCH(h, hipLaunchKernelGGL((moe_router_kernel<T>), dim3(T_), dim3(RF_THREADS), (size_t)W * sizeof(float), stream,
-      (const T*)h.data_ptr(), wr.data_ptr<float>(), W, rows, (int)E, (int)top, (int)groups, (int)keep, (float)scale,
-      ids.data_ptr<int>(), wts.data_ptr<float>(), extra.data_ptr<float>()));
+      (const T*)h.data_ptr(), wr.data_ptr<float>(), has_bias ? bias.data_ptr<float>() : nullptr, W, rows, (int)E,
+      (int)top, (int)groups, (int)keep, (float)scale, (int)score, ids.data_ptr<int>(), wts.data_ptr<float>(),
+      extra.data_ptr<float>()));
   return {ids, wts, extra};
 }
 
 // ---------------------------------------------------------------------------
-// y = g sigmoid(alpha g) (u + 1),  g = min(gate, limit), u = clamp(up, -limit, limit)
+// kind 0: y = g sigmoid(alpha g) (u + 1),  g = min(gate, limit), u = clamp(up, -limit, limit)
+// kind 1: y = gate sigmoid(gate) up
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void clamped_glu_kernel(const T* __restrict__ gu, long stride, T* __restrict__ y, long N, int F,
-                                   float limit, float alpha) {
+                                   float limit, float alpha, int kind) {
   const long total = N * F;
   for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
     const long n = i / F;
     const int f = (int)(i % F);
-    const float g = fminf(ldf(gu + n * stride + f), limit);
-    const float u = fminf(fmaxf(ldf(gu + n * stride + F + f), -limit), limit);
-    stf(y + i, g * sigmoidf_(alpha * g) * (u + 1.f));
+    float g = ldf(gu + n * stride + f), u = ldf(gu + n * stride + F + f);
+    if (kind == 0) {
+      g = fminf(g, limit);
+      u = fminf(fmaxf(u, -limit), limit);
+      stf(y + i, g * sigmoidf_(alpha * g) * (u + 1.f));
+    } else {
+      stf(y + i, g * sigmoidf_(g) * u);
+    }
   }
 }
 
-torch::Tensor clamped_glu(torch::Tensor gu, double limit, double alpha) {
+torch::Tensor clamped_glu(torch::Tensor gu, double limit, double alpha, int64_t kind) {
+  TORCH_CHECK(kind == 0 || kind == 1, "GLU kind: 0 clamped, 1 SiLU");
   TORCH_CHECK(gu.is_cuda() && gu.dim() == 2 && gu.stride(1) == 1 && gu.size(1) % 2 == 0);
   const long N = gu.size(0);
   const int F = gu.size(1) / 2;
@@ -305,7 +336,7 @@ torch::Tensor clamped_glu(torch::Tensor gu, double limit, double alpha) {
   if (N == 0) return y;
   auto stream = at::cuda::getCurrentHIPStream();
   RAGGED_DISPATCH(gu, hipLaunchKernelGGL((clamped_glu_kernel<T>), dim3(grid_for(N * F, 256)), dim3(256), 0, stream,
-      (const T*)gu.data_ptr(), (long)gu.stride(0), (T*)y.data_ptr(), N, F, (float)limit, (float)alpha));
+      (const T*)gu.data_ptr(), (long)gu.stride(0), (T*)y.data_ptr(), N, F, (float)limit, (float)alpha, (int)kind));
   return y;
 }
 

@@ -49,6 +49,19 @@ HYBRID_SRC = [
     "megatron_amd/ops/csrc/hybrid/delta_rule.hip",
 ]
 
+# the talking-heads models' extension carries the kernels it shares with the
+# other two through their sources, so a fresh checkout of such a model compiles
+# this extension alone
+TALKING_SRC = [
+    "megatron_amd/ops/csrc/talking/bindings.cpp",
+    "megatron_amd/ops/csrc/talking/depth_norm.hip",
+    "megatron_amd/ops/csrc/talking/talking_attention.hip",
+    "megatron_amd/ops/csrc/talking/talking_attention_mfma.hip",
+    "megatron_amd/ops/csrc/hybrid/rows.hip",
+    "megatron_amd/ops/csrc/hybrid/experts.hip",
+    "megatron_amd/ops/csrc/ragged/recurrent.hip",
+]
+
 # MEGATRON_AMD_ONLY_EXT=ragged builds just the serving kernels of the
 # ragged-batch models (what a fresh checkout compiles on first use); "hybrid"
 # likewise for the models built on the hybrid kernels
@@ -75,6 +88,12 @@ EXTS = {
         CUDAExtension(
             name="megatron_amd.ops._hybrid_ops",
             sources=HYBRID_SRC,
+            extra_compile_args={"cxx": ["-O3", "-std=c++17"], "nvcc": HIPCC_FLAGS},
+        ),
+    "talking": lambda:
+        CUDAExtension(
+            name="megatron_amd.ops._talking_ops",
+            sources=TALKING_SRC,
             extra_compile_args={"cxx": ["-O3", "-std=c++17"], "nvcc": HIPCC_FLAGS},
         ),
     "data": lambda:

@@ -1,0 +1,664 @@
+"""Tilarax model family: the framework's ragged engine path against a plain
+per-sequence oracle (tests/tilarax_oracle.py) on small random configurations.
+
+Covers each mechanism alone, prefill against token-by-token decoding, prompt
+portions down to two tokens, mixed batches against each request alone, reuse
+of freed pages and state slots, keys far away / at page borders / just inside
+and just outside a chunk (in prompts and in decoding, with a peaked softmax so
+that one key too many or too few shows), the first tokens of a sequence, long
+decoding, degenerate and unequal sizes, and greedy generation through the
+engine's own scheduler.
+"""
+
+import copy
+import json
+import math
+import os
+
+import pytest
+import torch
+
+import tilarax_oracle as O
+from megatron_amd.inference import DynamicInferenceEngine, SamplingParams
+from megatron_amd.inference.contexts import HybridInferenceContext
+from megatron_amd.models.tilarax import TilaraxConfig, TilaraxModel, load_tilarax_state
+
+F64 = torch.float64
+
+
+def attn(heads=4, kv=2, dim=6, vdim=5, chunk=7, rot=4, base=100.0, scale=0.6, v_mix=True, mlp="moe", experts=5,
+         top=2, ff=9):
+    m = dict(heads=heads, kv_heads=kv, dim=dim, vdim=vdim, scale=scale, v_mix=v_mix)
+    if chunk:
+        m["mask"] = dict(size=chunk)
+    if rot:
+        m["rot"] = dict(dims=rot, base=base)
+    return dict(type="attention", mixer=m, mlp=_mlp(mlp, experts, top, ff))
+
+
+def mlstm(heads=2, dim=5, vdim=7, cap=9.0, mlp="dense", experts=5, top=2, ff=11):
+    return dict(type="mlstm", mixer=dict(heads=heads, dim=dim, vdim=vdim, gate_cap=cap), mlp=_mlp(mlp, experts, top, ff))
+
+
+def _mlp(kind, experts, top, ff):
+    if kind is None:
+        return None
+    if kind == "dense":
+        return dict(kind="dense", ff=ff)
+    return dict(kind="moe", expert=dict(ff=ff), router=dict(experts=experts, top=top))
+
+
+def make_config(layers, width=24, vocab=41, eps=1e-5):
+    return dict(architecture="Tilarax", vocab=vocab, width=width, norm=dict(eps=eps), layers=copy.deepcopy(layers))
+
+
+def make_weights(cfg, seed=0, gain=1.0):
+    """Random checkpoint tensors under the checkpoint's names (bf16-representable
+    values so that both sides read the same numbers)."""
+    g = torch.Generator().manual_seed(seed)
+    W, out = cfg["width"], {}
+
+    def rnd(*shape, scale=1.0):
+        return (torch.randn(*shape, generator=g) * scale).to(torch.bfloat16).float()
+
+    def lin(o, i):
+        return rnd(o, i, scale=gain / math.sqrt(i))
+
+    out["embed"] = rnd(cfg["vocab"], W)
+    for i, L in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", L["mixer"]
+        a = p + "mix."
+        out[p + "norm1"] = rnd(W, scale=0.2)
+        if L["type"] == "attention":
+            H, G, d, e = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            out[a + "q"], out[a + "k"], out[a + "v"] = lin(H * d, W), lin(G * d, W), lin(G * e, W)
+            out[a + "q.b"], out[a + "k.b"], out[a + "v.b"] = rnd(H * d, scale=0.3), rnd(G * d, scale=0.3), rnd(G * e, scale=0.3)
+            out[a + "q.norm"], out[a + "k.norm"] = 1 + rnd(d, scale=0.2), 1 + rnd(d, scale=0.2)
+            out[a + "temp"] = 1 + rnd(H, scale=0.3).abs()
+            out[a + "talk"] = torch.eye(H) + rnd(H, H, scale=0.4)
+            out[a + "vmix"] = rnd(1).abs().clamp(0.2, 0.8).reshape(())
+            out[a + "o"], out[a + "o.b"] = lin(W, H * e), rnd(W, scale=0.3)
+        else:
+            H, d, e = m["heads"], m["dim"], m["vdim"]
+            out[a + "q"], out[a + "k"] = lin(H * d, W) * 2, lin(H * d, W) * 2
+            out[a + "v"], out[a + "g"], out[a + "o"] = lin(H * e, W), lin(H * e, W), lin(W, H * e)
+            out[a + "i"], out[a + "f"] = lin(H, W) * 3, lin(H, W) * 3
+            out[a + "i.b"], out[a + "f.b"] = rnd(H), rnd(H) + 2.0
+            out[a + "norm"] = 1 + rnd(H * e, scale=0.2)
+        if L.get("mlp"):
+            mm, q = L["mlp"], p + "mlp."
+            out[p + "norm2"] = rnd(W, scale=0.2)
+            if mm["kind"] == "dense":
+                out[q + "up"], out[q + "down"] = lin(mm["ff"], W) * 2, lin(W, mm["ff"])
+            else:
+                E, ff = mm["router"]["experts"], mm["expert"]["ff"]
+                out[q + "router"], out[q + "router.b"] = lin(E, W) * 3, rnd(E)
+                for e_ in range(E):
+                    out[f"{q}e{e_}.gate"], out[f"{q}e{e_}.up"], out[f"{q}e{e_}.down"] = lin(ff, W) * 2, lin(ff, W) * 2, lin(W, ff)
+        out[p + "dwa"] = rnd(i + 2, scale=0.3) + torch.cat([torch.zeros(i + 1), torch.ones(1)])
+    out["final.norm"] = rnd(W, scale=0.2)
+    return {k: v.to(torch.bfloat16).float() for k, v in out.items()}
+
+
+def build(cfg, weights, dtype=torch.float32, device="cpu"):
+    model = TilaraxModel(TilaraxConfig.from_dict(cfg, dtype=dtype))
+    load_tilarax_state(model, weights)
+    return model.to(device).eval()
+
+
+def engine_for(model, pages=40, page=8, slots=4, **kw):
+    return DynamicInferenceEngine(model, num_blocks=pages, block_size=page, max_batch=slots,
+                                  use_hip_graphs=False, enable_prefix_caching=False, **kw)
+
+
+def tokens_of(n, vocab, seed):
+    return torch.randint(0, vocab, (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+def feed(engine, req, toks):
+    """All positions' logits of one feed."""
+    return engine.forward_batch([(req, toks)], [list(range(len(toks)))])
+
+
+def assert_close(got, want, tol=2e-4):
+    want = want.float()
+    scale = want.abs().max().item()
+    err = (got.detach().cpu().float() - want).abs().max().item()
+    assert err <= tol * max(scale, 1.0), f"max abs error {err} (scale {scale})"
+
+
+def run_in_portions(engine, toks, cuts):
+    """Feed toks in portions of the given sizes (the rest one by one); all logits."""
+    req = engine.open_request()
+    out, at = [], 0
+    for c in cuts:
+        c = min(c, len(toks) - at)
+        if c <= 0:
+            break
+        out.append(feed(engine, req, toks[at:at + c]))
+        at += c
+    while at < len(toks):
+        out.append(feed(engine, req, toks[at:at + 1]))
+        at += 1
+    engine.close_request(req)
+    return torch.cat(out, dim=0)
+
+
+# attention first and last, two layers that mix values with the first, one that does not, a layer without feed-forward
+FULL = [mlstm(), attn(), mlstm(mlp="moe", dim=4), attn(heads=2, kv=2, dim=8, chunk=5, rot=8, mlp="dense"),
+        attn(v_mix=False, kv=1, vdim=3, chunk=11, rot=2, mlp=None), attn(heads=6, kv=2, dim=4, chunk=3, rot=0)]
+
+
+# -- each mechanism alone ------------------------------------------------------
+
+
+def test_post_norm_add_and_depth_history():
+    from megatron_amd.ops import ragged as R
+
+    torch.manual_seed(0)
+    T, W, L = 7, 24, 3
+    x0 = torch.randn(T, W)
+    x, hist = x0.clone(), torch.zeros(L + 1, T, W)
+    hist[0] = x0
+    ref_hist, cur = [x0.double()], x0.double()
+    for depth in range(1, L + 1):
+        y, y2, w, w2 = torch.randn(T, W) * 3, torch.randn(T, W), torch.randn(W) * 0.2, torch.randn(W) * 0.2
+        dwa = torch.randn(depth + 1)
+        h = R.post_norm_add(x, y, w, 1e-5, torch.float32)
+        cur = cur + O.norm_one_plus(y.double(), w.double(), 1e-5)
+        assert_close(h, cur, 1e-5)
+        h = R.post_norm_add(x, y2, w2, 1e-5, torch.float32, hist, depth, dwa)
+        cur = cur + O.norm_one_plus(y2.double(), w2.double(), 1e-5)
+        ref_hist.append(cur)
+        cur = sum(dwa[j].double() * ref_hist[j] for j in range(depth + 1))
+        assert_close(h, cur, 1e-5)
+        assert_close(x, cur, 1e-5)
+        assert_close(hist[depth], ref_hist[depth], 1e-5)
+
+
+def _module_ctx(caches, states, n, page, dtype=torch.float32, device="cpu"):
+    pages = (n + page - 1) // page
+    ctx = HybridInferenceContext(caches, states, pages + 2, page, 2, dtype=dtype, device=device)
+    ctx.allocator.allocate(1)
+    table = ctx.allocator.allocate(pages)[::-1]
+    return ctx, table, ctx.acquire_slot()
+
+
+def _attention_weights(W, H, G, D, V, seed):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=g)     # noqa: E731
+    return {"q": r(H * D, W) / 4, "k": r(G * D, W) / 4, "v": r(G * V, W) / 4, "q.b": r(H * D) / 3, "k.b": r(G * D) / 3,
+            "v.b": r(G * V) / 3, "q.norm": 1 + 0.2 * r(D), "k.norm": 1 + 0.2 * r(D), "temp": 1 + r(H).abs(),
+            "talk": torch.eye(H) + 0.5 * r(H, H), "vmix": torch.tensor(0.35), "o": r(W, H * V) / 4, "o.b": r(W) / 3}
+
+
+def _attention_module(W, m, wt, eps=1e-5):
+    from megatron_amd.transformer.talking_heads_attention import TalkingHeadsAttention
+
+    rot = m.get("rot") or {}
+    mod = TalkingHeadsAttention(W, m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["scale"], eps,
+                                rot_dims=rot.get("dims", 0), rot_base=rot.get("base", 1.0),
+                                chunk=(m.get("mask") or {}).get("size"), value_mix=m.get("v_mix", False),
+                                dtype=torch.float32)
+    with torch.no_grad():
+        mod.w_in.copy_(torch.cat([wt["q"], wt["k"], wt["v"]]))
+        mod.b_in.copy_(torch.cat([wt["q.b"], wt["k.b"], wt["v.b"]]))
+        mod.q_norm.copy_(wt["q.norm"]); mod.k_norm.copy_(wt["k.norm"]); mod.temp.copy_(wt["temp"])
+        mod.talk.copy_(wt["talk"]); mod.lam.copy_(wt["vmix"].reshape(1)); mod.w_out.copy_(wt["o"]); mod.b_out.copy_(wt["o.b"])
+    return mod
+
+
+@pytest.mark.parametrize("H,G,D,V,chunk,rot", [(4, 2, 6, 5, 7, 4), (3, 3, 4, 4, 1, 4), (2, 1, 8, 3, 13, 0), (4, 4, 4, 6, None, 2),
+                                               (6, 2, 2, 2, 64, 2), (1, 1, 10, 1, 8, 6), (4, 1, 5, 4, 9, 4)])
+@pytest.mark.parametrize("mix", [False, True])
+def test_attention_alone(H, G, D, V, chunk, rot, mix):
+    torch.manual_seed(1)
+    W, n, page = 16, 45, 8
+    m = dict(heads=H, kv_heads=G, dim=D, vdim=V, scale=1.5, v_mix=mix)
+    if chunk:
+        m["mask"] = dict(size=chunk)
+    if rot:
+        m["rot"] = dict(dims=rot, base=50.0)
+    wt = _attention_weights(W, H, G, D, V, 3)
+    mod = _attention_module(W, m, wt)
+    h = torch.randn(n, W)
+    v_first = torch.randn(n, G, V) if mix else None
+    want, _ = O.attention_mixer(h.double(), m, {k: v.double() for k, v in wt.items()}, "", 1e-5,
+                                v_first.double() if mix else None)
+    ctx, table, slot = _module_ctx(mod.cache_spec("a", page), {}, n, page)
+    got, at = [], 0
+    for c in (19, 2, 1, 13, 10):                      # portions: every chunk edge is cut somewhere
+        ctx.begin_batch([c], [at], [slot], [table])
+        carry = {"v_first": v_first[at:at + c].reshape(c, G * V)} if mix else {}
+        with torch.no_grad():
+            got.append(mod(h[at:at + c], ctx, "a", carry))
+        at += c
+    assert at == n
+    assert_close(torch.cat(got), want, 1e-5)
+
+
+def test_first_mixing_layer_keeps_its_values_and_hands_them_on():
+    torch.manual_seed(2)
+    W, n = 16, 9
+    m = dict(heads=2, kv_heads=1, dim=4, vdim=3, scale=1.0, v_mix=True, mask=dict(size=4))
+    wt = _attention_weights(W, 2, 1, 4, 3, 4)
+    mod = _attention_module(W, m, wt)
+    h = torch.randn(n, W)
+    want, v = O.attention_mixer(h.double(), m, {k: x.double() for k, x in wt.items()}, "", 1e-5, None)
+    ctx, table, slot = _module_ctx(mod.cache_spec("a", 8), {}, n, 8)
+    ctx.begin_batch([n], [0], [slot], [table])
+    carry = {}
+    with torch.no_grad():
+        got = mod(h, ctx, "a", carry)
+    assert_close(got, want, 1e-5)
+    assert_close(carry["v_first"], v.reshape(n, 3), 1e-5)       # unmixed, whatever its own lam
+
+
+@pytest.mark.parametrize("H,D,V,cap", [(2, 5, 7, 9.0), (1, 8, 3, 2.0), (3, 4, 4, 30.0)])
+def test_mlstm_alone(H, D, V, cap):
+    from megatron_amd.ssm.mlstm import MLSTMMixer
+
+    torch.manual_seed(3)
+    W, n = 16, 33
+    g = lambda *s: torch.randn(*s)     # noqa: E731
+    wt = {"q": g(H * D, W) / 2, "k": g(H * D, W) / 2, "v": g(H * V, W) / 4, "g": g(H * V, W) / 4, "o": g(W, H * V) / 4,
+          "i": g(H, W), "f": g(H, W), "i.b": g(H), "f.b": g(H) + 2, "norm": 1 + 0.2 * g(H * V)}
+    mod = MLSTMMixer(W, H, D, V, cap, 1e-5, "s", dtype=torch.float32)
+    with torch.no_grad():
+        mod.w_in.copy_(torch.cat([wt[k] for k in "qkvg"]))
+        mod.w_gates.copy_(torch.cat([wt["i"], wt["f"]]))
+        mod.bias_i.copy_(wt["i.b"]); mod.bias_f.copy_(wt["f.b"]); mod.norm_weight.copy_(wt["norm"]); mod.w_out.copy_(wt["o"])
+    h = torch.randn(n, W)
+    want = O.mlstm_mixer(h.double(), dict(heads=H, dim=D, vdim=V, gate_cap=cap), {k: v.double() for k, v in wt.items()}, "", 1e-5)
+    ctx, table, slot = _module_ctx({}, mod.state_spec(), n, 8)
+    got, at = [], 0
+    for c in (17, 1, 2, 13):
+        ctx.begin_batch([c], [at], [slot], [table])
+        with torch.no_grad():
+            got.append(mod(h[at:at + c], ctx))
+        at += c
+    assert_close(torch.cat(got), want, 2e-5)
+
+
+def test_mlstm_running_maximum_starts_at_zero():
+    """With strongly negative input gates the stabiliser stays at its start value 0 (not at the
+    gates' level): the read-out's denominator is then max(|n.q|, 1), which shows in the output."""
+    from megatron_amd.ops import ragged_reference as ref
+
+    H, D, V = 1, 2, 2
+    qkvg = torch.tensor([[1.0, 0.0, 1.0, 0.0, 2.0, 4.0, 30.0, 30.0]])
+    gates = torch.tensor([[-5.0, 40.0]])          # log input gate -5, forget gate ~ 0
+
+    class B:
+        num_requests, host_cu, host_start, host_slots = 1, [0, 1], [0], [0]
+    S, n, m = torch.zeros(1, 1, D, V), torch.zeros(1, 1, D), torch.zeros(1, 1)
+    ref.mlstm_scan(qkvg, gates, torch.zeros(1), torch.zeros(1), torch.ones(2), H, D, V, 50.0, 0.0, S, n, m, B, torch.float32)
+    assert abs(m.item()) < 1e-6                    # max(f + 0, i) = f ~ 0, not i
+    i = 50.0 * math.tanh(-5.0 / 50.0)
+    assert_close(S[0, 0, 0] / math.exp(i), torch.tensor([2.0, 4.0]), 1e-5)
+
+
+@pytest.mark.parametrize("E,top", [(6, 2), (8, 1), (5, 5), (9, 3)])
+def test_router_alone(E, top):
+    from megatron_amd.ops import ragged as R
+
+    torch.manual_seed(3)
+    h, wr, br = torch.randn(50, 16), torch.randn(E, 16), torch.randn(E) * 2
+    idx, wt = O.route(h.double(), dict(experts=E, top=top), {"router": wr.double(), "router.b": br.double()}, "")
+    ids, w, _ = R.moe_router(h, wr, E, top, 1, 1, 1.0, br, "softmax")
+    o1, o2 = idx.argsort(1), ids.long().argsort(1)
+    assert torch.equal(idx.gather(1, o1), ids.long().gather(1, o2))
+    assert_close(w.gather(1, o2), wt.gather(1, o1), 1e-6)
+    assert_close(w.sum(1), torch.ones(50), 1e-6)
+
+
+def test_router_bias_decides():
+    """A bias far above the logits' spread picks its expert whatever the token is."""
+    from megatron_amd.ops import ragged as R
+
+    torch.manual_seed(4)
+    h, wr = torch.randn(20, 16), torch.randn(4, 16)
+    br = torch.tensor([0.0, 0.0, 100.0, 0.0])
+    ids, w, _ = R.moe_router(h, wr, 4, 1, 1, 1, 1.0, br, "softmax")
+    assert (ids == 2).all() and (w == 1).all()
+
+
+@pytest.mark.parametrize("kind", ["dense", "moe"])
+def test_feed_forward_alone(kind):
+    cfg = make_config([mlstm(mlp=kind)])
+    w = make_weights(cfg, seed=4)
+    layer = build(cfg, w).layers[0]
+    torch.manual_seed(5)
+    h = torch.randn(21, cfg["width"])
+    with torch.no_grad():
+        got = layer.mlp(h)
+    assert_close(got, O.feed_forward(h.double(), cfg["layers"][0]["mlp"], {k: v.double() for k, v in w.items()}, "l0.mlp."), 1e-5)
+
+
+@pytest.mark.parametrize("spec", [attn(), attn(mlp=None), attn(kv=4, mlp="dense"), attn(kv=1, chunk=1), attn(chunk=None),
+                                  attn(rot=6, top=5), attn(rot=0, top=1), mlstm(), mlstm(mlp="moe"), mlstm(mlp=None, heads=1)],
+                         ids=["attn", "attn-no-ff", "mha-dense", "mqa-chunk1", "no-chunks", "rot-all-top-all", "no-rot-top1",
+                              "mlstm", "mlstm-moe", "mlstm-no-ff"])
+def test_single_layer_matches_oracle(spec):
+    cfg = make_config([spec])
+    w = make_weights(cfg, seed=1)
+    toks = tokens_of(37, cfg["vocab"], 2)
+    got = build(cfg, w)(torch.tensor([toks]))[:, 0]
+    assert_close(got, O.forward(cfg, w, toks))
+
+
+# -- whole model through the engine -------------------------------------------------
+
+
+def test_layers_match_oracle():
+    cfg = make_config(FULL)
+    w = make_weights(cfg, seed=6)
+    toks = tokens_of(40, cfg["vocab"], 7)
+    model = build(cfg, w)
+    model.layer_trace = []
+    eng = engine_for(model)
+    req = eng.open_request()
+    got = feed(eng, req, toks)
+    trace = []
+    want = O.forward(cfg, w, toks, F64, trace)
+    assert len(model.layer_trace) == len(trace) == len(FULL)
+    for a, b in zip(model.layer_trace, trace):
+        assert_close(a, b)
+    assert_close(got, want)
+    spec = model.inference_spec(8)
+    assert set(spec.caches) == {"l1", "l3", "l4", "l5"} and {"l0.mlstm.S", "l2.mlstm.S"} <= set(spec.states)
+
+
+def test_prefill_then_decode_token_by_token():
+    cfg = make_config(FULL)
+    w = make_weights(cfg, seed=8)
+    toks = tokens_of(48, cfg["vocab"], 9)
+    want = O.forward(cfg, w, toks)
+    eng = engine_for(build(cfg, w))
+    assert_close(run_in_portions(eng, toks, [20]), want)          # 20 at once, then 28 single tokens
+    assert_close(run_in_portions(eng, toks, []), want)            # everything token by token
+
+
+@pytest.mark.parametrize("cuts", [[2, 2, 2, 3, 5, 2, 17, 2], [7, 1, 1, 9, 4, 4, 11], [31, 2], [3] * 16])
+def test_portions(cuts):
+    cfg = make_config(FULL)
+    w = make_weights(cfg, seed=10)
+    toks = tokens_of(47, cfg["vocab"], 11)
+    eng = engine_for(build(cfg, w))
+    assert_close(run_in_portions(eng, toks, cuts), O.forward(cfg, w, toks))
+
+
+def test_mixed_batch_equals_each_alone():
+    cfg = make_config(FULL)
+    w = make_weights(cfg, seed=12)
+    model = build(cfg, w)
+    seqs = [tokens_of(n, cfg["vocab"], 20 + n) for n in (29, 7, 18, 3)]
+    want = [O.forward(cfg, w, s) for s in seqs]
+    eng = engine_for(model, pages=12)
+    reqs = [eng.open_request() for _ in seqs]
+    at = [0] * len(seqs)
+    got = [[] for _ in seqs]
+    plan = [(5, 1, 2, 3), (2, 1, 0, 0), (1, 1, 7, 0), (9, 1, 1, 0), (1, 1, 1, 0), (11, 2, 7, 0)]
+    for step in plan:
+        feeds, wants, who = [], [], []
+        for r, c in enumerate(step):
+            c = min(c, len(seqs[r]) - at[r])
+            if c > 0:
+                feeds.append((reqs[r], seqs[r][at[r]:at[r] + c]))
+                wants.append(list(range(c)))
+                who.append((r, c))
+                at[r] += c
+        out = eng.forward_batch(feeds, wants)
+        o = 0
+        for r, c in who:
+            got[r].append(out[o:o + c])
+            o += c
+    for r in range(len(seqs)):
+        assert at[r] == len(seqs[r])
+        assert_close(torch.cat(got[r]), want[r])
+
+
+def test_freed_pages_and_slots_are_reused():
+    cfg = make_config(FULL)
+    w = make_weights(cfg, seed=13)
+    eng = engine_for(build(cfg, w), pages=5, page=8, slots=2)     # room for one 40-token request at a time
+    for seed in (30, 31, 32):
+        toks = tokens_of(33 + seed % 3, cfg["vocab"], seed)
+        assert_close(run_in_portions(eng, toks, [9, 2, 12]), O.forward(cfg, w, toks))
+    a, b = eng.open_request(), eng.open_request()                 # both slots, used before
+    ta, tb = tokens_of(11, cfg["vocab"], 40), tokens_of(17, cfg["vocab"], 41)
+    out = eng.forward_batch([(a, ta), (b, tb)], [list(range(11)), list(range(17))])
+    assert_close(out[:11], O.forward(cfg, w, ta))
+    assert_close(out[11:], O.forward(cfg, w, tb))
+
+
+# -- edges -----------------------------------------------------------------------------
+
+
+def _peaked():
+    """One attention layer whose softmax is peaked (large scale): a key too many or too few moves the output."""
+    return make_config([attn(heads=2, kv=1, dim=8, vdim=6, chunk=5, rot=4, scale=6.0, mlp=None, v_mix=False)])
+
+
+def test_one_key_more_or_less_shows():
+    cfg = _peaked()
+    w = make_weights(cfg, seed=14)
+    toks = tokens_of(30, cfg["vocab"], 15)
+    a = O.forward(cfg, w, toks)
+    other = copy.deepcopy(cfg)
+    other["layers"][0]["mixer"]["mask"]["size"] = 6
+    b = O.forward(other, w, toks)
+    assert (a - b).abs().max().item() > 50 * 2e-4 * a.abs().max().item()
+
+
+@pytest.mark.parametrize("page", [4, 8])
+def test_chunk_edges_at_every_offset_to_page_borders(page):
+    """chunk 5 against pages of 4 or 8: walking 45 positions puts a chunk's first and last position at every
+    offset to a page border; decoded one by one, in portions of two, and in one piece"""
+    cfg = _peaked()
+    w = make_weights(cfg, seed=14)
+    toks = tokens_of(45, cfg["vocab"], 16)
+    want = O.forward(cfg, w, toks)
+    model = build(cfg, w)
+    for cuts in ([], [2] * 22, [45], [4, 1, 5, 6, 4, 10]):
+        eng = engine_for(model, pages=16, page=page)
+        assert_close(run_in_portions(eng, toks, cuts), want)
+
+
+def _planted(n, chunk, H, G, D, V, target, seed):
+    """q, k, v of one sequence in which the LAST query matches the key at ``target`` far better than any other"""
+    g = torch.Generator().manual_seed(seed)
+    q, k, v = torch.randn(n, H, D, generator=g), torch.randn(n, G, D, generator=g), torch.randn(n, G, V, generator=g)
+    rep = H // G
+    for hd in range(H):
+        q[n - 1, hd] = 6.0 * k[target, hd // rep] / k[target, hd // rep].norm()
+    k[target] *= 3.0
+    return q, k, v
+
+
+@pytest.mark.parametrize("n,chunk,target,seen", [(300, 0, 0, True), (300, 512, 3, True), (290, 97, 194, True), (290, 97, 193, False),
+                                                 (65, 64, 64, True), (65, 64, 63, False), (130, 64, 128, True), (130, 64, 127, False)])
+@pytest.mark.parametrize("decode", [False, True])
+def test_far_and_edge_keys_in_the_attention_op(n, chunk, target, seen, decode):
+    """a key far back among hundreds, at a page border, and just inside / outside the chunk of the last
+    query, which is either the end of a prompt portion or a token decoded alone"""
+    from megatron_amd.ops import ragged as R
+
+    H, G, D, V, page = 4, 2, 8, 5, 16
+    q, k, v = _planted(n, chunk, H, G, D, V, target, 5)
+    temp, talk = torch.ones(H), torch.eye(H) + 0.1
+    want = O.talking_softmax_attention(q.double(), k.double(), v.double(), 1.0, temp.double(), talk.double(), chunk or None)
+    ctx, table, slot = _module_ctx({"c": G * (D + V)}, {}, n, page)
+    rows = torch.cat([k.reshape(n, -1), v.reshape(n, -1)], dim=1)
+    cuts = [n - 1, 1] if decode else [n - 40, 40]
+    at, got = 0, []
+    for c in cuts:
+        batch = ctx.begin_batch([c], [at], [slot], [table])
+        ctx.pools["c"][batch.tok_row] = rows[at:at + c]
+        got.append(R.talking_attention(q[at:at + c].reshape(c, -1), ctx.pools["c"], H, G, D, V, 1.0, temp, talk, chunk,
+                                       batch, torch.float32))
+        at += c
+    got = torch.cat(got)
+    assert_close(got, want, 1e-5)
+    # the planted key dominates the last row exactly when it is visible
+    last = got[-1].view(H, V)
+    own = torch.stack([talk[hd].sum() * v[target, hd // (H // G)] for hd in range(H)])
+    assert ((last - own).abs().max().item() < 0.15) == seen
+
+
+@pytest.mark.parametrize("n", [1, 2, 3])
+def test_first_tokens(n):
+    cfg = make_config(FULL)
+    w = make_weights(cfg, seed=17)
+    toks = tokens_of(n, cfg["vocab"], 18)
+    eng = engine_for(build(cfg, w))
+    assert_close(run_in_portions(eng, toks, [n]), O.forward(cfg, w, toks))
+    assert_close(run_in_portions(eng, toks, []), O.forward(cfg, w, toks))
+
+
+def test_long_decoding():
+    cfg = make_config(FULL)
+    w = make_weights(cfg, seed=19)
+    toks = tokens_of(100, cfg["vocab"], 20)
+    eng = engine_for(build(cfg, w), pages=14)
+    assert_close(run_in_portions(eng, toks, [5]), O.forward(cfg, w, toks), 3e-4)
+
+
+@pytest.mark.parametrize("layers,width,vocab", [
+    ([attn(heads=1, kv=1, dim=2, vdim=1, chunk=2, rot=2, experts=1, top=1, ff=1)], 8, 5),
+    ([attn(v_mix=False), attn(v_mix=True, mlp="dense"), attn(v_mix=True, chunk=4), attn(v_mix=True, chunk=64)], 16, 30),
+    ([mlstm(mlp=None), mlstm(heads=3, dim=3, vdim=2, mlp="moe", experts=3, top=3)], 12, 17),
+    ([attn(heads=8, kv=4, dim=4, vdim=4, rot=4, chunk=16, experts=2, top=2), mlstm(heads=4, dim=4, vdim=4, cap=1.0)], 32, 64),
+], ids=["all-ones", "mixing-starts-late", "only-mlstm", "equal-sizes"])
+def test_other_sizes(layers, width, vocab):
+    cfg = make_config(layers, width=width, vocab=vocab)
+    w = make_weights(cfg, seed=21)
+    toks = tokens_of(29, vocab, 22)
+    eng = engine_for(build(cfg, w))
+    assert_close(run_in_portions(eng, toks, [6, 2, 9]), O.forward(cfg, w, toks))
+
+
+# -- entry points ----------------------------------------------------------------------
+
+
+def test_greedy_generation_through_the_scheduler():
+    cfg = make_config(FULL)
+    w = make_weights(cfg, seed=23)
+    model = build(cfg, w)
+    prompts = [tokens_of(n, cfg["vocab"], 50 + n) for n in (13, 4, 21, 9, 2)]   # more requests than slots
+    eng = engine_for(model, pages=16, slots=3, max_prefill_tokens=10)            # prompts go in in portions
+    res = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=7, stop_on_eod=False))
+    for p, r in zip(prompts, res):
+        seq = list(p)
+        for tok in r.output_tokens:
+            logits = O.forward(cfg, w, seq)[-1]
+            top2 = logits.topk(2).values
+            if (top2[0] - top2[1]).item() > 1e-3:                                # a near-tie may go either way
+                assert tok == int(logits.argmax())
+            seq.append(tok)
+        assert len(r.output_tokens) == 7
+
+
+def test_registry_builds_from_a_directory(tmp_path):
+    from safetensors.torch import save_file
+
+    from megatron_amd.models.registry import build_from_dir
+
+    cfg = make_config(FULL)
+    w = make_weights(cfg, seed=24)
+    with open(os.path.join(tmp_path, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    save_file({k: v.to(torch.bfloat16).contiguous() for k, v in w.items()}, os.path.join(tmp_path, "model.safetensors"))
+    model = build_from_dir(str(tmp_path), dtype=torch.float32)
+    toks = tokens_of(20, cfg["vocab"], 25)
+    assert_close(model(torch.tensor([toks]))[:, 0], O.forward(cfg, w, toks))
+
+
+def test_trace_replay(tmp_path):
+    """the replay runner drives the same step function: two requests fed in unequal portions, one ended early"""
+    import io
+
+    from megatron_amd.inference.trace import replay
+
+    cfg = make_config(FULL)
+    w = make_weights(cfg, seed=26)
+    eng = engine_for(build(cfg, w))
+    a, b = tokens_of(12, cfg["vocab"], 27), tokens_of(9, cfg["vocab"], 28)
+    steps = [dict(step=0, entries=[dict(id="a", tokens=a[:7], want=[6]), dict(id="b", tokens=b[:2], want=[])], end=[]),
+             dict(step=1, entries=[dict(id="b", tokens=b[2:], want=[0, 6])], end=["b"]),
+             dict(step=2, entries=[dict(id="a", tokens=a[7:], want=[4])], end=["a"])]
+    log = io.StringIO()
+    replay(eng, [json.dumps(s) for s in steps], str(tmp_path), log)
+    assert log.getvalue().split() == ["done", "0", "done", "1", "done", "2"]
+    import numpy as np
+
+    V = cfg["vocab"]
+    r0 = torch.from_numpy(np.fromfile(os.path.join(tmp_path, "0.f32"), dtype="<f4").reshape(-1, V))
+    r1 = torch.from_numpy(np.fromfile(os.path.join(tmp_path, "1.f32"), dtype="<f4").reshape(-1, V))
+    r2 = torch.from_numpy(np.fromfile(os.path.join(tmp_path, "2.f32"), dtype="<f4").reshape(-1, V))
+    wa, wb = O.forward(cfg, w, a), O.forward(cfg, w, b)
+    assert_close(r0, wa[6:7]); assert_close(r1, wb[[2, 8]]); assert_close(r2, wa[11:12])
+
+
+# -- the HIP path ------------------------------------------------------------------------
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("cuts", [[40], [13, 2, 1, 9], []])
+def test_gpu_fp32_matches_oracle(cuts):
+    cfg = make_config(FULL)
+    w = make_weights(cfg, seed=6)
+    toks = tokens_of(40, cfg["vocab"], 7)
+    eng = engine_for(build(cfg, w, device="cuda"))
+    assert_close(run_in_portions(eng, toks, cuts), O.forward(cfg, w, toks))
+
+
+@pytest.mark.gpu
+def test_gpu_fp32_mixed_batch_and_reuse():
+    cfg = make_config(FULL)
+    w = make_weights(cfg, seed=12)
+    eng = engine_for(build(cfg, w, device="cuda"), pages=9, slots=2)
+    for round_ in range(2):                                         # the second round reuses pages and slots
+        a, b = tokens_of(30, cfg["vocab"], 60 + round_), tokens_of(11, cfg["vocab"], 70 + round_)
+        ra, rb = eng.open_request(), eng.open_request()
+        o1 = eng.forward_batch([(ra, a[:17]), (rb, b[:1])], [list(range(17)), [0]])
+        o2 = eng.forward_batch([(ra, a[17:18]), (rb, b[1:])], [[0], list(range(10))])
+        o3 = eng.forward_batch([(ra, a[18:])], [list(range(12))])
+        eng.close_request(ra); eng.close_request(rb)
+        assert_close(torch.cat([o1[:17], o2[:1], o3]), O.forward(cfg, w, a))
+        assert_close(torch.cat([o1[17:], o2[1:]]), O.forward(cfg, w, b))
+
+
+@pytest.mark.gpu
+def test_gpu_bf16_close_to_oracle():
+    """bf16 storage with fp32 residual, norms, scores and state; routing takes every expert so that
+    rounding cannot flip a close choice; head sizes that run on the matrix cores"""
+    layers = [mlstm(dim=8, vdim=8), attn(dim=16, vdim=8, rot=8, chunk=7, experts=3, top=3),
+              attn(heads=2, kv=2, dim=8, vdim=8, chunk=5, rot=8, mlp="dense"), mlstm(mlp="moe", experts=2, top=2)]
+    cfg = make_config(layers, width=32)
+    w = make_weights(cfg, seed=31)
+    toks = tokens_of(44, cfg["vocab"], 32)
+    want = O.forward(cfg, w, toks)
+    eng = engine_for(build(cfg, w, dtype=torch.bfloat16, device="cuda"))
+    for cuts in ([44], [9, 2, 20], []):
+        got = run_in_portions(eng, toks, cuts).float().cpu()
+        d = got - want.float()
+        err = (d - d.mean(-1, keepdim=True)).pow(2).mean(-1).sqrt().max().item()
+        assert err < 0.06 * want.float().std().item() + 0.05, err
+
+
+@pytest.mark.gpu
+def test_gpu_greedy_generation():
+    cfg = make_config(FULL)
+    w = make_weights(cfg, seed=23)
+    prompts = [tokens_of(n, cfg["vocab"], 50 + n) for n in (13, 4, 21)]
+    eng = engine_for(build(cfg, w, device="cuda"), pages=16, slots=2, max_prefill_tokens=10)
+    res = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=5, stop_on_eod=False))
+    for p, r in zip(prompts, res):
+        seq = list(p)
+        for tok in r.output_tokens:
+            logits = O.forward(cfg, w, seq)[-1]
+            top2 = logits.topk(2).values
+            if (top2[0] - top2[1]).item() > 1e-3:
+                assert tok == int(logits.argmax())
+            seq.append(tok)

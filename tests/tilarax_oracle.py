@@ -54,11 +54,27 @@ def chunk_mask(T, size):
     return (j <= i) & (torch.div(i, size, rounding_mode="floor") == torch.div(j, size, rounding_mode="floor"))
 
 
+def talking_softmax_attention(q, k, v, scale, temp, talk, size):
+    """q [T, H, d], k [T, G, d], v [T, G, e] of one whole sequence -> [T, H * e].
+    Dense: every head's softmax over the visible keys, the weights mixed over
+    the heads by ``talk``, head h then reads the values of its own key/value head."""
+    T, H = q.shape[0], q.shape[1]
+    rep = H // k.shape[1]
+    mask = chunk_mask(T, size) if size else chunk_mask(T, T)
+    probs = []
+    for hd in range(H):
+        s = (q[:, hd] @ k[:, hd // rep].T) * scale * temp[hd]
+        s = s.masked_fill(~mask, float("-inf"))
+        probs.append(torch.softmax(s, dim=-1))
+    mixed = torch.einsum("hg,gij->hij", talk, torch.stack(probs))
+    return torch.cat([mixed[hd] @ v[:, hd // rep] for hd in range(H)], dim=-1)
+
+
 def attention_mixer(h, m, w, p, eps, v_first):
     """h [T, W]; m the layer's mixer config; w tensors; p the tensor prefix.
     -> (output [T, W], the values this layer caches [T, G, e])"""
     T = h.shape[0]
-    H, G, d, e = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    H, G, d, e = m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m["vdim"]
     q = (h @ w[p + "q"].T + w[p + "q.b"]).view(T, H, d)
     k = (h @ w[p + "k"].T + w[p + "k.b"]).view(T, G, d)
     v = (h @ w[p + "v"].T + w[p + "v.b"]).view(T, G, e)
@@ -72,17 +88,8 @@ def attention_mixer(h, m, w, p, eps, v_first):
     if m.get("v_mix") and v_first is not None:
         lam = w[p + "vmix"]
         v = (1.0 - lam) * v + lam * v_first
-    rep = H // G
-    mask = chunk_mask(T, m["mask"]["size"])
-    probs = []
-    for hd in range(H):
-        s = (q[:, hd] @ k[:, hd // rep].T) * m["scale"] * w[p + "temp"][hd]
-        s = s.masked_fill(~mask, float("-inf"))
-        probs.append(torch.softmax(s, dim=-1))
-    probs = torch.stack(probs)                       # [H, T, T]
-    mixed = torch.einsum("hg,gij->hij", w[p + "talk"], probs)
-    outs = [mixed[hd] @ v[:, hd // rep] for hd in range(H)]
-    o = torch.cat(outs, dim=-1)                      # [T, H * e]
+    size = (m.get("mask") or {}).get("size")
+    o = talking_softmax_attention(q, k, v, m["scale"], w[p + "temp"], w[p + "talk"], size)
     return o @ w[p + "o"].T + w[p + "o.b"], v
 
 
