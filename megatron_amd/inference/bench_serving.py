@@ -13,6 +13,11 @@ one prompt per prefill step, batched decode steps).  One JSON line per
 beside a delta-rule memory, routed experts) next to the Bezutar design with
 alternating attention / mLSTM layers at the same width, depth and active
 feed-forward size, both through the same ragged engine path.
+
+``--serve-design tilarax`` measures the Tilarax design (mLSTM layers alternating
+with chunked talking-heads attention layers, post-sublayer norms with a
+depth-weighted residual history, dense and routed feed-forwards in turn) next
+to the same Bezutar pattern.
 """
 
 from __future__ import annotations
@@ -75,6 +80,28 @@ def bezurax_config(size):
                 logit_scale=1.0, layers=[json.loads(json.dumps(one)) for _ in range(s["layers"])])
 
 
+# Tilarax at the same widths and depths: mLSTM layers (the sizes above) with a dense feed-forward
+# alternate with attention layers of query heads x 128, a quarter as many kv heads, chunks of
+# 1024 positions, half of every head rotated, values mixed with the first attention layer's, and
+# 16 experts of which 4 are chosen: the active feed-forward size equals the dense ff above
+T_SIZES = {
+    "1b": dict(heads=16, kv=4, dim=128, chunk=1024, rot=64, experts=16, top=4, eff=1408),
+    "7b-layers": dict(heads=32, kv=8, dim=128, chunk=1024, rot=64, experts=16, top=4, eff=2752),
+}
+
+
+def tilarax_config(size):
+    s, x = SIZES[size], T_SIZES[size]
+    rec = dict(type="mlstm", mixer=dict(heads=s["m_heads"], dim=s["m_dim"], vdim=s["m_vdim"], gate_cap=15.0),
+               mlp=dict(kind="dense", ff=s["ff"]))
+    att = dict(type="attention",
+               mixer=dict(heads=x["heads"], kv_heads=x["kv"], dim=x["dim"], vdim=x["dim"], scale=x["dim"] ** -0.5,
+                          mask=dict(size=x["chunk"]), rot=dict(base=10000.0, dims=x["rot"]), v_mix=True),
+               mlp=dict(kind="moe", expert=dict(ff=x["eff"]), router=dict(experts=x["experts"], top=x["top"])))
+    layers = [json.loads(json.dumps(att if i % 2 else rec)) for i in range(s["layers"])]
+    return dict(architecture="Tilarax", vocab=s["vocab"], width=s["width"], norm=dict(eps=1e-6), layers=layers)
+
+
 def _random_init(model, seed=0):
     g = torch.Generator(device="cpu").manual_seed(seed)
     with torch.no_grad():
@@ -86,6 +113,13 @@ def _random_init(model, seed=0):
                 p.copy_(torch.randn(p.shape, generator=g) * p.shape[-1] ** -0.5)
             elif name.endswith("weight") and p.dim() == 2:      # canon taps
                 p.copy_(torch.randn(p.shape, generator=g) * 0.2)
+            elif name.endswith(".dwa"):                         # mostly the layer's own result
+                p.fill_(0.1)
+                p[-1] = 1.0
+            elif name.endswith(".talk"):
+                p.add_((torch.randn(p.shape, generator=g) * 0.1).to(p.device))
+            elif name.endswith(".lam"):
+                p.fill_(0.3)
 
 
 def _time(fn):
@@ -116,6 +150,16 @@ def run_bezurax(size, batch, isl, osl, device):
         model = BezuraxModel(cfg).eval()
     _random_init(model)
     return _run_ragged(model, "bezurax", size, batch, isl, osl, device)
+
+
+def run_tilarax(size, batch, isl, osl, device):
+    from megatron_amd.models.tilarax import TilaraxConfig, TilaraxModel
+
+    cfg = TilaraxConfig.from_dict(tilarax_config(size), dtype=torch.bfloat16)
+    with torch.device(device):
+        model = TilaraxModel(cfg).eval()
+    _random_init(model)
+    return _run_ragged(model, "tilarax", size, batch, isl, osl, device)
 
 
 def _run_ragged(model, label, size, batch, isl, osl, device):
@@ -206,8 +250,10 @@ def main(args) -> None:
     device = torch.device("cuda", 0)
     torch.cuda.set_device(0)
     for size in args.serve_sizes.split(","):
-        if getattr(args, "serve_design", "bezutar") == "bezurax":
-            r = run_bezurax(size, args.serve_batch, args.serve_isl, args.serve_osl, device)
+        design = getattr(args, "serve_design", "bezutar")
+        if design in ("bezurax", "tilarax"):
+            run = run_bezurax if design == "bezurax" else run_tilarax
+            r = run(size, args.serve_batch, args.serve_isl, args.serve_osl, device)
             r.update(batch=args.serve_batch, isl=args.serve_isl, osl=args.serve_osl, dtype="bf16", data="synthetic")
             print(json.dumps(r), flush=True)
             torch.cuda.empty_cache()
