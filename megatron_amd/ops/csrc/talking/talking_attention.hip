@@ -185,6 +185,19 @@ __global__ __launch_bounds__(256) void talk_mix_kernel(const float* __restrict__
   const long t = blockIdx.x;
   const int rep = H / G;
   const float* At = A + t * H * G * V;
+  if (V % 4 == 0) {                              // 16 B reads of A
+    const int V4 = V / 4;
+    for (int i = threadIdx.x; i < H * V4; i += 256) {
+      const int h = i / V4, d = (i % V4) * 4, c = h / rep;
+      float4v a = float4v{0.f, 0.f, 0.f, 0.f};
+      for (int g = 0; g < H; ++g)
+        a += s_talk[h * H + g] * *reinterpret_cast<const float4v*>(At + ((long)g * G + c) * V + d);
+      T* op = out + t * H * V + (long)h * V + d;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) stf(op + k, a[k]);
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < H * V; i += 256) {
     const int h = i / V, d = i % V, c = h / rep;
     float a = 0.f;
