@@ -5,11 +5,16 @@
 // so this kernel computes A for every query head g and EVERY value head c, in
 // fp32, and talk_mix_kernel (talking_attention.hip) forms the sums.
 //
+// The value heads lie side by side in a cache row, so A[g, c0 .. c0+CG-1] is ONE
+// product with a value CG * V wide: a workgroup takes as many value heads as its
+// accumulators hold (up to 512 columns), and the scores and the softmax are
+// computed once per group of CG value heads instead of once per value head.
+//
 // Rows of the problem are (token, query head) pairs of ONE request and ONE key
 // head (the rep = H / G query heads that share it), 64 per workgroup (16 per
-// wave), numbered token-major; blockIdx.z = key head * G + value head picks the
-// key columns and the value columns of the cache row that are staged, in tiles
-// of 32 positions, as [key | value] in LDS.  A row at position p sees
+// wave), numbered token-major; blockIdx.z = key head * groups + value group picks
+// the key columns and the value columns of the cache row that are staged, in
+// tiles of 32 positions, as [key | values] in LDS.  A row at position p sees
 // positions chunk_start(p) .. p, chunk_start(p) = floor(p / chunk) * chunk
 // (0 without chunks); the tiles run from the chunk start of the workgroup's
 // FIRST token to its last token and the rest of a tile is masked per row.
@@ -44,7 +49,8 @@ __global__ __launch_bounds__(256) void talking_attn_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ pool, float scale, const float* __restrict__ temp,
     int chunk, const int* __restrict__ tiles, const int* __restrict__ cu, const int* __restrict__ start_pos,
     const int* __restrict__ tables, int maxb, int bs, float* __restrict__ out, float* __restrict__ part_o,
-    float* __restrict__ part_m, float* __restrict__ part_l, int nsplit, int Tn, int H, int G, int D, int V) {
+    float* __restrict__ part_m, float* __restrict__ part_l, int nsplit, int Tn, int H, int G, int D, int V,
+    int CG) {
   static_assert(NT % 4 == 0, "value tiles are dealt to four waves");
   constexpr int NTW = NT / 4;                    // value tiles per wave
   constexpr int KW = NKS * 32;                   // staged key columns (zero-padded)
@@ -53,7 +59,10 @@ __global__ __launch_bounds__(256) void talking_attn_mfma_kernel(
   short* const p_lds = lds + TK_KT * ldk;
   float* const f_lds = reinterpret_cast<float*>(p_lds + TK_ROWS * TK_KT);
   const int req = tiles[2 * blockIdx.x], row0 = tiles[2 * blockIdx.x + 1];
-  const int kvh = blockIdx.z / G, vh = blockIdx.z % G, rep = H / G;
+  const int NVG = (G + CG - 1) / CG;              // groups of value heads
+  const int kvh = blockIdx.z / NVG, vg = blockIdx.z % NVG, rep = H / G;
+  const int vcol0 = vg * CG * V;                  // first value column of the group, among the G * V of a row
+  const int VW = min(CG, G - vg * CG) * V;        // its width
   const int t0 = cu[req], n_rows = (cu[req + 1] - t0) * rep, start = start_pos[req];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g4 = lane >> 4;
   const int width = G * (D + V);
@@ -121,8 +130,8 @@ __global__ __launch_bounds__(256) void talking_attn_mfma_kernel(
     int col = -1;
     if (d < KW) {
       if (d < D) col = kvh * D + d;
-    } else if (d - KW < V) {
-      col = G * D + vh * V + (d - KW);
+    } else if (d - KW < VW) {
+      col = G * D + vcol0 + (d - KW);
     }
     s_col[k] = (i < TK_KT * cpr) ? col : -1;
   }
@@ -262,46 +271,48 @@ __global__ __launch_bounds__(256) void talking_attn_mfma_kernel(
       const int row = row0 + rt * 16 + c;
       if (row < n_rows) {
         const float inv = f_lds[rt * 16 + c];
-        float* op = out + (((long)(t0 + row / rep) * H + kvh * rep + row % rep) * G + vh) * V;
+        float* op = out + ((long)(t0 + row / rep) * H + kvh * rep + row % rep) * G * V + vcol0;
 #pragma unroll
         for (int i = 0; i < NTW; ++i) {
           const int d = (wave + 4 * i) * 16 + 4 * g4;
-          if (d < V) *reinterpret_cast<f32x4*>(op + d) = oacc[i][rt] * inv;
+          if (d < VW) *reinterpret_cast<f32x4*>(op + d) = oacc[i][rt] * inv;
         }
       }
     }
   } else {
-    const long rows_all = (long)Tn * H * G;
+    const long rows_all = (long)Tn * H;
     if (g4 == 0 && row_ok) {
-      const long grow = ((long)(t0 + my_tok) * H + my_head) * G + vh;
-      part_m[blockIdx.y * rows_all + grow] = m;
-      part_l[blockIdx.y * rows_all + grow] = l;
+      const long grow = (long)(t0 + my_tok) * H + my_head;
+      part_m[(blockIdx.y * rows_all + grow) * NVG + vg] = m;
+      part_l[(blockIdx.y * rows_all + grow) * NVG + vg] = l;
     }
 #pragma unroll
     for (int rt = 0; rt < 4; ++rt) {
       const int row = row0 + rt * 16 + c;
       if (row < n_rows) {
-        const long grow = ((long)(t0 + row / rep) * H + kvh * rep + row % rep) * G + vh;
-        float* po = part_o + (blockIdx.y * rows_all + grow) * V;
+        const long grow = (long)(t0 + row / rep) * H + kvh * rep + row % rep;
+        float* po = part_o + (blockIdx.y * rows_all + grow) * G * V + vcol0;
 #pragma unroll
         for (int i = 0; i < NTW; ++i) {
           const int d = (wave + 4 * i) * 16 + 4 * g4;
-          if (d < V) *reinterpret_cast<f32x4*>(po + d) = oacc[i][rt];
+          if (d < VW) *reinterpret_cast<f32x4*>(po + d) = oacc[i][rt];
         }
       }
     }
   }
 }
 
-// merge of the key splits: one workgroup per (token, query head, value head) row of A
+// merge of the key splits: one workgroup per (token, query head, value head) row of A;
+// rows = tokens * heads, the statistics are kept per (row, group of value heads)
 __global__ void talking_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_m,
                                        const float* __restrict__ part_l, float* __restrict__ out, int nsplit,
-                                       long rows, int V) {
+                                       long rows, int G, int V, int CG) {
   __shared__ float s_m[TK_MAX_SPLIT], s_l[TK_MAX_SPLIT];
-  const long grow = blockIdx.x;
+  const long grow = blockIdx.x / G;
+  const int c = blockIdx.x % G, NVG = (G + CG - 1) / CG, vg = c / CG;
   if (threadIdx.x < nsplit) {
-    s_m[threadIdx.x] = part_m[threadIdx.x * rows + grow];
-    s_l[threadIdx.x] = part_l[threadIdx.x * rows + grow];
+    s_m[threadIdx.x] = part_m[(threadIdx.x * rows + grow) * NVG + vg];
+    s_l[threadIdx.x] = part_l[(threadIdx.x * rows + grow) * NVG + vg];
   }
   __syncthreads();
   float M = TK_NEG;
@@ -312,8 +323,8 @@ __global__ void talking_combine_kernel(const float* __restrict__ part_o, const f
   for (int d = threadIdx.x; d < V; d += blockDim.x) {
     float a = 0.f;
 #pragma unroll 4
-    for (int s = 0; s < nsplit; ++s) a += part_o[(s * rows + grow) * V + d] * expf(s_m[s] - M);
-    out[grow * V + d] = a * inv;
+    for (int s = 0; s < nsplit; ++s) a += part_o[((s * rows + grow) * G + c) * V + d] * expf(s_m[s] - M);
+    out[(grow * G + c) * V + d] = a * inv;
   }
 }
 
@@ -328,7 +339,7 @@ torch::Tensor talking_attention_mfma(torch::Tensor q, torch::Tensor pool, int64_
   check_i32(tiles, "tiles"); check_i32(cu, "cu"); check_i32(start_pos, "start_pos"); check_i32(tables, "tables");
   check_f32(temp, "temp"); check_f32(talk, "talk");
   const int T_ = q.size(0), R = start_pos.numel();
-  TORCH_CHECK(G >= 1 && H % G == 0 && bs >= 1 && chunk >= 0 && G * G <= 65535);
+  TORCH_CHECK(G >= 1 && H % G == 0 && bs >= 1 && chunk >= 0 && G * G <= 65535 && (long)T_ * H * G < (1L << 31));
   TORCH_CHECK(temp.numel() == H && talk.numel() == H * H);
   TORCH_CHECK(D % 8 == 0 && V % 8 == 0 && D <= 256 && V <= 256, "MFMA path: head dims multiples of 8, at most 256");
   TORCH_CHECK(pool.size(0) % bs == 0);
@@ -337,6 +348,11 @@ torch::Tensor talking_attention_mfma(torch::Tensor q, torch::Tensor pool, int64_
   auto out = torch::empty({T_, H * V}, q.options());
   const int nblk = tiles.size(0);
   if (T_ == 0 || nblk == 0) return out;
+  // value heads per workgroup: as many as the widest instantiation for this key size holds
+  const int nks = ((int)D + 31) / 32;
+  const int wide = nks <= 4 ? 512 : 256;
+  const int CG = std::max(1, std::min((int)G, wide / (int)V));
+  const int NVG = ((int)G + CG - 1) / CG, nt = (CG * (int)V + 15) / 16;
   auto fo = q.options().dtype(at::kFloat);
   auto A = torch::empty({(long)T_ * H * G, V}, fo);      // every row is written by a workgroup or the combine
   auto stream = at::cuda::getCurrentHIPStream();
@@ -344,26 +360,26 @@ torch::Tensor talking_attention_mfma(torch::Tensor q, torch::Tensor pool, int64_
   float *pop = nullptr, *pmp = nullptr, *plp = nullptr;
   if (nsplit > 1) {
     po = torch::empty({nsplit, (long)T_ * H * G, V}, fo);
-    pm = torch::empty({nsplit, (long)T_ * H * G}, fo);
-    pl = torch::empty({nsplit, (long)T_ * H * G}, fo);
+    pm = torch::empty({nsplit, (long)T_ * H * NVG}, fo);
+    pl = torch::empty({nsplit, (long)T_ * H * NVG}, fo);
     pop = po.data_ptr<float>(); pmp = pm.data_ptr<float>(); plp = pl.data_ptr<float>();
   }
-  const dim3 grid(nblk, (unsigned)nsplit, (unsigned)(G * G));
+  const dim3 grid(nblk, (unsigned)nsplit, (unsigned)(G * NVG));
 #define TK_MFMA(NKS, NT)                                                                                        \
   hipLaunchKernelGGL((talking_attn_mfma_kernel<NKS, NT>), grid, dim3(256),                                      \
       ((size_t)TK_KT * (NKS * 32 + NT * 16 + 8) + TK_ROWS * TK_KT) * sizeof(short) + TK_ROWS * sizeof(float),   \
       stream, (const bf16*)q.data_ptr(), (const bf16*)pool.data_ptr(), (float)scale, temp.data_ptr<float>(),    \
       (int)chunk, tiles.data_ptr<int>(), cu.data_ptr<int>(), start_pos.data_ptr<int>(), tables.data_ptr<int>(), \
       (int)tables.size(1), (int)bs, A.data_ptr<float>(), pop, pmp, plp, (int)nsplit, T_, (int)H, (int)G,        \
-      (int)D, (int)V)
-  const int nks = ((int)D + 31) / 32, nt = ((int)V + 15) / 16;
+      (int)D, (int)V, CG)
   if (nks <= 2 && nt <= 4) TK_MFMA(2, 4);
   else if (nks <= 4 && nt <= 8) TK_MFMA(4, 8);
+  else if (nks <= 4) TK_MFMA(4, 32);
   else TK_MFMA(8, 16);
 #undef TK_MFMA
   if (nsplit > 1)
     hipLaunchKernelGGL(talking_combine_kernel, dim3((unsigned)((long)T_ * H * G)), dim3(128), 0, stream, pop, pmp,
-                       plp, A.data_ptr<float>(), (int)nsplit, (long)T_ * H * G, (int)V);
+                       plp, A.data_ptr<float>(), (int)nsplit, (long)T_ * H, (int)G, (int)V, CG);
   talk_mix_launch(A, talk, out, (int)H, (int)G, (int)V);
   return out;
 }

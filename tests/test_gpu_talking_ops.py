@@ -78,11 +78,13 @@ def test_head_norm_rope_store(dtype, shape, mix):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape", [(4, 2, 24, 24, 9), (3, 3, 80, 40, 0), (6, 1, 144, 144, 64), (2, 2, 16, 8, 1),
-                                   (8, 2, 64, 64, 40), (2, 1, 12, 20, 5), (4, 4, 32, 48, 200), (1, 1, 256, 256, 33)])
+                                   (8, 2, 64, 64, 40), (2, 1, 12, 20, 5), (4, 4, 32, 48, 200), (1, 1, 256, 256, 33),
+                                   (8, 4, 32, 64, 40), (3, 3, 16, 200, 30), (2, 2, 160, 128, 50), (16, 8, 128, 128, 100)])
 @pytest.mark.parametrize("starts", [STARTS, [0, 300, 130, 3, 517]], ids=["short", "long"])
 def test_talking_attention(dtype, shape, starts):
     """heads, kv heads, dim, vdim, chunk (0: none); page 16: chunks cross pages and page borders
-    lie inside chunks; long contexts beside short ones make the bf16 kernel split the key tiles"""
+    lie inside chunks; long contexts beside short ones make the bf16 kernel split the key tiles; the
+    last shapes make a workgroup take several value heads, an uneven last group, and wide keys"""
     R = _need()
     H, G, D, V, chunk = shape
 
