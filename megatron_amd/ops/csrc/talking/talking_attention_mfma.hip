@@ -353,7 +353,7 @@ torch::Tensor talking_attention_mfma(torch::Tensor q, torch::Tensor pool, int64_
   const int wide = nks <= 4 ? 512 : 256;          // measured: 512 columns beat 256 and 128 at 128-wide heads
   int CG = std::max(1, std::min((int)G, wide / (int)V));
   // steps with few rows (decoding) keep one value head a workgroup: more workgroups, shorter ones
-  if ((long)nblk * G * ((G + CG - 1) / CG) * nsplit < 512) CG = 1;
+  if ((long)nblk * G * ((G + CG - 1) / CG) < 256) CG = 1;
   const int NVG = ((int)G + CG - 1) / CG, nt = (CG * (int)V + 15) / 16;
   auto fo = q.options().dtype(at::kFloat);
   auto A = torch::empty({(long)T_ * H * G, V}, fo);      // every row is written by a workgroup or the combine
