@@ -386,7 +386,7 @@ def moe_router(h, w_router, experts, top, groups, keep, scale, bias=None, score=
     score "sigmoid": sigmoid scores, group-limited choice, weights = chosen scores / their sum * scale;
     score "softmax": the largest logits are chosen, weights = softmax over the chosen logits."""
     ext = _pick(h, "hybrid", "talking")
-    if ext is not None and h.shape[1] <= 15360 and w_router.shape[0] <= 512:
+    if ext is not None and h.shape[1] <= 15360 and w_router.shape[0] <= 512 and top <= 16 and groups <= 64:
         return ext.moe_router(h, w_router, bias if bias is not None else _none(h.device), int(experts), int(top),
                               int(groups), int(keep), float(scale), ROUTER_SCORES[score])
     return ref.moe_router(h, w_router, experts, top, groups, keep, scale, bias, score)

@@ -26,9 +26,11 @@ def _need():
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("ydtype", [torch.float32, torch.bfloat16])
-def test_post_norm_add_and_depth_history(dtype, ydtype):
+@pytest.mark.parametrize("W", [200, 202, 1027])
+def test_post_norm_add_and_depth_history(dtype, ydtype, W):
+    """widths that are and are not a multiple of four (the kernel's wide accesses), above one pass of a workgroup"""
     R = _need()
-    T, W, L = 13, 200, 3
+    T, L = 13, 3
 
     def run(dev, dt):
         x = _rand((T, W), torch.float32, dev)
