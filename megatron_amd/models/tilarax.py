@@ -111,6 +111,7 @@ class TilaraxModel(nn.Module):
         self.embedding = nn.Parameter(torch.zeros(config.vocab_size, W, dtype=dt))   # also the output matrix
         self.layers = nn.ModuleList([TilaraxLayer(config, i) for i in range(config.num_layers)])
         self.final_norm_weight = nn.Parameter(torch.zeros(W, dtype=torch.float32))   # applied as 1 + w
+        self.register_buffer("_one", torch.ones(1, dtype=torch.float32), persistent=False)
         self.layer_trace: Optional[list] = None   # debugging: what every layer hands on
 
     # -- what the cache/state manager must provide ------------------------------
@@ -132,8 +133,7 @@ class TilaraxModel(nn.Module):
         dt, eps, L = cfg.params_dtype, cfg.norm_eps, cfg.num_layers
         x = R.embed_plain(tokens, self.embedding)                  # [T, W] fp32 residual
         hist = torch.empty(L + 1, *x.shape, dtype=torch.float32, device=x.device)
-        hist[0].copy_(x)
-        h = x if dt == torch.float32 else x.to(dt)
+        h = R.post_norm_add(x, None, None, eps, dt, hist, 0, self._one)   # X_0 into the history, x in the GEMM dtype
         carry: dict = {}                                           # lives for this step (first mixed values)
         for i, layer in enumerate(self.layers):
             y = layer.mix(h, ctx, carry)
