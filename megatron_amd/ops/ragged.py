@@ -434,7 +434,10 @@ def talking_attention(q, pool, heads, kv_heads, dim, vdim, scale, temp, talk, ch
             # matrix-core kernel: 64 (token, head-in-group) rows per workgroup and (key head, group of
             # value heads) pair; steps with few rows (decode) also split the key tiles over workgroups
             tiles = batch.row_tiles(heads // kv_heads, q.device)
-            nblk = tiles.shape[0] * kv_heads * max(1, (kv_heads * vdim + 511) // 512)
+            groups = max(1, (kv_heads * vdim + 511) // 512)
+            if tiles.shape[0] * kv_heads * groups < 256:      # the kernel's rule: one value head a workgroup
+                groups = kv_heads
+            nblk = tiles.shape[0] * kv_heads * groups
             keys = min(batch.max_context, chunk) if chunk > 0 else batch.max_context
             nsplit = max(1, min((keys + 63) // 64, 1024 // max(nblk, 1), 64))
             return _K.talking_attention_mfma(q, pool, int(heads), int(kv_heads), int(dim), int(vdim), float(scale),
