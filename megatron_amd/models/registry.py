@@ -66,6 +66,13 @@ def _tilarax(path, dtype, device):
     return build_tilarax_from_dir(path, dtype=dtype, device=device)
 
 
+@register_model("Lomazen")
+def _lomazen(path, dtype, device):
+    from megatron_amd.models.lomazen import build_lomazen_from_dir
+
+    return build_lomazen_from_dir(path, dtype=dtype, device=device)
+
+
 @register_model("LlamaForCausalLM")
 def _llama(path, dtype, device):
     """HuggingFace Llama checkpoints -> GPTModel (single process, TP=1)."""

@@ -10,7 +10,10 @@ Expert (no biases): g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit),
 y = g sigmoid(alpha g) (u + 1), output W_down y.
 Other designs choose by the raw logits and weigh by the softmax over the chosen
 logits (``score="softmax"``, optional router bias), and use the plain SiLU GLU
-y = g sigmoid(g) u (``activation="silu"``).
+y = g sigmoid(g) u (``activation="silu"``).  ``score="softmax_all"`` chooses the largest
+logits and weighs them by their softmax over ALL experts (the weights do not
+sum to one); ``activation="relu2"`` makes experts WITHOUT a gate matrix,
+W_down relu(W_up h)^2 (``w_up`` [experts, ff, hidden] in place of ``w_gate_up``).
 Optional shared expert of the same form for every token, times
 sigmoid(w_sg . h); its gate row rides in the fp32 router GEMM.
 
@@ -42,7 +45,9 @@ class RoutedExpertsMLP(nn.Module):
                  shared_limit: Optional[float] = None, alpha: float = 1.702, score: str = "sigmoid",
                  router_bias: bool = False, activation: str = "clamped", dtype=torch.bfloat16):
         super().__init__()
-        assert score in R.ROUTER_SCORES and activation in R.GLU_KINDS
+        assert score in R.ROUTER_SCORES and (activation in R.GLU_KINDS or activation == "relu2")
+        self.gated = activation != "relu2"
+        assert self.gated or not shared_ff, "the shared expert is a GLU"
         assert score == "sigmoid" or groups <= 1, "group-limited choice is defined on sigmoid scores"
         self.score, self.activation = score, activation
         assert top <= experts and experts % max(groups, 1) == 0
@@ -56,7 +61,10 @@ class RoutedExpertsMLP(nn.Module):
         self.w_router = nn.Parameter(torch.zeros(experts + (1 if shared_ff else 0), hidden, dtype=torch.float32))
         self.b_router = (nn.Parameter(torch.zeros(experts + (1 if shared_ff else 0), dtype=torch.float32))
                          if router_bias else None)
-        self.w_gate_up = nn.Parameter(torch.zeros(experts, 2 * ff, hidden, dtype=dtype))   # [gate; up] per expert
+        if self.gated:
+            self.w_gate_up = nn.Parameter(torch.zeros(experts, 2 * ff, hidden, dtype=dtype))   # [gate; up] per expert
+        else:
+            self.w_up = nn.Parameter(torch.zeros(experts, ff, hidden, dtype=dtype))
         self.w_down = nn.Parameter(torch.zeros(experts, hidden, ff, dtype=dtype))
         if shared_ff:
             self.ws_gate_up = nn.Parameter(torch.zeros(2 * shared_ff, hidden, dtype=dtype))
@@ -68,6 +76,8 @@ class RoutedExpertsMLP(nn.Module):
                             self.b_router, self.score)
 
     def _glu(self, gu, limit, dtype):
+        if not self.gated:
+            return R.relu2(gu, dtype)
         return R.glu(gu, self.activation, limit, self.alpha, dtype)
 
     def _grouped_ok(self, h: torch.Tensor) -> bool:
@@ -88,7 +98,10 @@ class RoutedExpertsMLP(nn.Module):
             gate = extra.reshape(-1)
         if R.expert_pairs_ok(h, K, self.ff):
             # few pairs (decoding): each pair streams its expert's matrices, no sort, no host read
-            down = R.expert_pairs(h, ids, self.w_gate_up, self.w_down, self.limit, self.alpha, self.activation)
+            if self.gated:
+                down = R.expert_pairs(h, ids, self.w_gate_up, self.w_down, self.limit, self.alpha, self.activation)
+            else:
+                down = R.expert_pairs_plain(h, ids, self.w_up, self.w_down)
             inv = torch.arange(T * K, dtype=torch.int32, device=h.device).view(T, K)
             return R.moe_combine(down, inv, weights, shared, gate, add)
         flat = ids.reshape(-1).long()
@@ -96,10 +109,11 @@ class RoutedExpertsMLP(nn.Module):
         inv = torch.empty_like(order)
         inv[order] = torch.arange(order.numel(), device=order.device)
         xs = h.index_select(0, torch.div(order, K, rounding_mode="floor"))
+        w_first = self.w_gate_up if self.gated else self.w_up
         if self._grouped_ok(h):
             # one grouped GEMM per linear over the sorted pairs, group ends on the device: no host read
             offs = torch.cumsum(torch.bincount(flat, minlength=E), 0).to(torch.int32)
-            gu = torch._grouped_mm(xs, self.w_gate_up.transpose(1, 2), offs=offs)
+            gu = torch._grouped_mm(xs, w_first.transpose(1, 2), offs=offs)
             down = torch._grouped_mm(self._glu(gu, self.limit, h.dtype),
                                      self.w_down.transpose(1, 2), offs=offs)
         else:
@@ -108,7 +122,7 @@ class RoutedExpertsMLP(nn.Module):
             at = 0
             for e, n in enumerate(counts):
                 if n:
-                    gu = F.linear(xs[at:at + n], self.w_gate_up[e])
+                    gu = F.linear(xs[at:at + n], w_first[e])
                     down[at:at + n] = F.linear(self._glu(gu, self.limit, h.dtype), self.w_down[e])
                     at += n
         return R.moe_combine(down, inv.view(T, K).to(torch.int32), weights, shared, gate, add)

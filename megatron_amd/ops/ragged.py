@@ -13,6 +13,12 @@ per-head q/k norm with pairwise rotation, value mixing and cache store, chunked
 talking-heads attention, tanh-GELU; it also carries the embedding, mLSTM and
 routed-expert kernels of the other two (same sources), so that a model built
 on it compiles nothing else.
+``_gated_ops``: norms on both sides of a sublayer, restart of a repeated block
+of layers, rotation in pairs or halves with an optional unit norm and cache
+store, attention with one or two softmax maps a head (capped scores; gated or
+differential finish), squared ReLU, experts without a gate matrix; it carries
+the embedding, final-norm, router, GLU and expert kernels of ``_hybrid_ops``
+(same sources).
 
 Dispatch rule (same as megatron_amd.ops): tensors on a HIP device run the
 CDNA4 kernels of the extension (csrc/ragged/*.hip, csrc/hybrid/*.hip) and RAISE
@@ -34,17 +40,18 @@ from megatron_amd.ops.ragged_reference import rope_table  # noqa: F401  (host-si
 _C = None      # _ragged_ops: latent attention, mLSTM, minGRU, hyper-connections, canon conv, xIELU
 _H = None      # _hybrid_ops: grouped norm, pooled-window attention, delta rule, routed experts
 _K = None      # _talking_ops: post-norm with depth history, talking-heads attention (+ shared kernels)
+_G = None      # _gated_ops: sandwich norms, capped / differential attention (+ shared kernels)
 _IMPORT_ERROR: Optional[str] = None
 _IMPORT_ERRORS = {}
 
 # setup.py extension key -> module name; a model names the keys it needs in
 # ``native_extensions`` and a serving process builds only those on first use
-EXTENSIONS = {"ragged": "_ragged_ops", "hybrid": "_hybrid_ops", "talking": "_talking_ops"}
+EXTENSIONS = {"ragged": "_ragged_ops", "hybrid": "_hybrid_ops", "talking": "_talking_ops", "gated": "_gated_ops"}
 
 
 def _load(key: str = "ragged"):
-    global _C, _H, _K, _IMPORT_ERROR
-    cur = {"ragged": _C, "hybrid": _H, "talking": _K}[key]
+    global _C, _H, _K, _G, _IMPORT_ERROR
+    cur = {"ragged": _C, "hybrid": _H, "talking": _K, "gated": _G}[key]
     if cur is not None:
         return cur
     try:
@@ -55,8 +62,10 @@ def _load(key: str = "ragged"):
             _C = mod
         elif key == "hybrid":
             _H = mod
-        else:
+        elif key == "talking":
             _K = mod
+        else:
+            _G = mod
         return mod
     except Exception as e:  # noqa: BLE001
         _IMPORT_ERRORS[key] = repr(e)
@@ -68,6 +77,7 @@ def _load(key: str = "ragged"):
 _load("ragged")
 _load("hybrid")
 _load("talking")
+_load("gated")
 
 
 def build_extension(key: str, verbose: bool = False) -> None:
@@ -130,7 +140,7 @@ def _pick(x: torch.Tensor, *keys):
     if not x.is_cuda or os.environ.get("MEGATRON_AMD_FORCE_REFERENCE", "0") == "1":
         return None
     for key in keys:
-        mod = {"ragged": _C, "hybrid": _H, "talking": _K}[key]
+        mod = {"ragged": _C, "hybrid": _H, "talking": _K, "gated": _G}[key]
         if mod is not None:
             return mod
     raise RuntimeError(
@@ -257,7 +267,7 @@ def gate_heads(x, gate_pre, heads):
 
 
 def embed_plain(tokens, embed):
-    ext = _pick(embed, "hybrid", "talking")
+    ext = _pick(embed, "hybrid", "talking", "gated")
     if ext is not None:
         return ext.embed_plain(tokens, embed)
     return ref.embed_plain(tokens, embed)
@@ -265,7 +275,7 @@ def embed_plain(tokens, embed):
 
 def residual_group_norm(x, y, w_a, w_b, groups, eps, out_dtype):
     """x fp32 [T, W] += y in place (y may be None); -> (norm(x) w_a, norm(x) w_b or None)."""
-    ext = _pick(x, "hybrid", "talking")
+    ext = _pick(x, "hybrid", "talking", "gated")
     if ext is not None:
         d = x.device
         h_a, h_b = ext.residual_group_norm(x, y if y is not None else _none(d), w_a,
@@ -331,7 +341,7 @@ def moe_route(logits, experts, top, groups, keep, scale):
     return ref.moe_route(logits, experts, top, groups, keep, scale)
 
 
-GLU_KINDS = {"clamped": 0, "silu": 1}
+GLU_KINDS = {"clamped": 0, "silu": 1, "gelu_tanh": 2}
 
 
 def clamped_glu(gu, limit, alpha, out_dtype):
@@ -340,17 +350,19 @@ def clamped_glu(gu, limit, alpha, out_dtype):
 
 def glu(gu, act, limit, alpha, out_dtype):
     """gu [N, 2F] = [gate | up] -> [N, F]: "clamped": min(g, limit) sigmoid(alpha g) (clamp(u) + 1);
-    "silu": g sigmoid(g) u."""
-    ext = _pick(gu, "hybrid", "talking")
+    "silu": g sigmoid(g) u; "gelu_tanh": gelu_tanh(g) u."""
+    ext = _pick(gu, "hybrid", "talking", "gated")
     if ext is not None:
         return ext.clamped_glu(gu, float(limit), float(alpha), GLU_KINDS[act])
     if act == "silu":
         return ref.silu_glu(gu, out_dtype)
+    if act == "gelu_tanh":
+        return ref.gelu_glu(gu, out_dtype)
     return ref.clamped_glu(gu, limit, alpha, out_dtype)
 
 
 def moe_combine(down, inv, weights, shared, shared_gate, add):
-    ext = _pick(down, "hybrid", "talking")
+    ext = _pick(down, "hybrid", "talking", "gated")
     if ext is not None:
         d = down.device
         return ext.moe_combine(down, inv, weights, shared if shared is not None else _none(d),
@@ -364,28 +376,29 @@ PAIR_PATH_MAX = 32      # (token, choice) pairs up to which every pair streams i
 
 def expert_pairs_ok(h, top, ff) -> bool:
     """Steps with few pairs (decoding) skip the sort by expert: see csrc/hybrid/experts.hip."""
-    return (h.is_cuda and (_H is not None or _K is not None)
+    return (h.is_cuda and (_H is not None or _K is not None or _G is not None)
             and os.environ.get("MEGATRON_AMD_FORCE_REFERENCE", "0") != "1"
             and h.shape[0] * top <= PAIR_PATH_MAX and h.shape[1] % 8 == 0 and ff % 8 == 0
             and max(h.shape[1], ff) <= 15360)
 
 
 def expert_pairs(h, ids, w_gate_up, w_down, limit, alpha, act="clamped"):
-    ext = _pick(h, "hybrid", "talking")
+    ext = _pick(h, "hybrid", "talking", "gated")
     if ext is not None:
         return ext.expert_pairs(h, ids, w_gate_up, w_down, float(limit), float(alpha), GLU_KINDS[act])
     return ref.expert_pairs(h, ids, w_gate_up, w_down, limit, alpha, act)
 
 
-ROUTER_SCORES = {"sigmoid": 0, "softmax": 1}
+ROUTER_SCORES = {"sigmoid": 0, "softmax": 1, "softmax_all": 2}
 
 
 def moe_router(h, w_router, experts, top, groups, keep, scale, bias=None, score="sigmoid"):
     """-> (ids [T, top] int32, weights [T, top] fp32, raw logits of the rows beyond the experts)
 
     score "sigmoid": sigmoid scores, group-limited choice, weights = chosen scores / their sum * scale;
-    score "softmax": the largest logits are chosen, weights = softmax over the chosen logits."""
-    ext = _pick(h, "hybrid", "talking")
+    score "softmax": the largest logits are chosen, weights = softmax over the chosen logits;
+    score "softmax_all": the largest logits are chosen, weights = their softmax over ALL experts."""
+    ext = _pick(h, "hybrid", "talking", "gated")
     if ext is not None and h.shape[1] <= 15360 and w_router.shape[0] <= 512 and top <= 16 and groups <= 64:
         return ext.moe_router(h, w_router, bias if bias is not None else _none(h.device), int(experts), int(top),
                               int(groups), int(keep), float(scale), ROUTER_SCORES[score])
@@ -453,3 +466,110 @@ def gelu_tanh(z, out_dtype):
     if _native_k(z):
         return _K.gelu_tanh(z)
     return ref.gelu_tanh(z, out_dtype)
+
+
+# ---------------------------------------------------------------------------
+# ops of the gated extension: norms on both sides of a sublayer, restart of a
+# repeated block of layers, rotation (pairs / halves) with unit norm and cache
+# store, attention with one or two softmax maps a head, gated and differential
+# finish, squared ReLU, experts without a gate matrix
+# ---------------------------------------------------------------------------
+
+scaled_freqs = ref.scaled_freqs
+ROT_LAYOUTS = ref.ROT_LAYOUTS
+
+
+def _native_g(x: torch.Tensor) -> bool:
+    return _pick(x, "gated") is not None
+
+
+def sandwich_norm_add(x, y, w_post, w_pre, eps, out_dtype, copy_to=None):
+    """x fp32 [T, W] <- x + rms_unit(y) w_post in place (y may be None); ``copy_to`` (a [T, W]
+    view of any row stride) receives the new x; -> rms_unit(x) w_pre in out_dtype, or None."""
+    if _native_g(x):
+        d = x.device
+        h = _G.sandwich_norm_add(x, y if y is not None else _none(d), w_post if y is not None else _none(d),
+                                 w_pre if w_pre is not None else _none(d), float(eps), out_dtype == torch.bfloat16,
+                                 copy_to if copy_to is not None else _none(d))
+        return h if w_pre is not None else None
+    return ref.sandwich_norm_add(x, y, w_post, w_pre, eps, out_dtype, copy_to)
+
+
+def restart_norm(y, bias, w_pre, eps, out_dtype):
+    """-> (x fp32 = y + bias, rms_unit(x) w_pre in out_dtype)"""
+    if _native_g(y):
+        x, h = _G.restart_norm(y, bias, w_pre, float(eps), out_dtype == torch.bfloat16)
+        return x, h
+    return ref.restart_norm(y, bias, w_pre, eps, out_dtype)
+
+
+def rope_norm_store(proj, q_heads, k_heads, dim, v_width, freqs, layout, unit_norm, eps, pool, batch):
+    if _native_g(proj):
+        return _G.rope_norm_store(proj, int(q_heads), int(k_heads), int(dim), int(v_width), freqs,
+                                  ROT_LAYOUTS[layout], bool(unit_norm), float(eps), pool, batch.tok_pos,
+                                  batch.tok_row)
+    return ref.rope_norm_store(proj, q_heads, k_heads, dim, v_width, freqs, layout, unit_norm, eps, pool, batch)
+
+
+def _map_mfma_ok(q, dim, vdim) -> bool:
+    return (q.dtype == torch.bfloat16 and dim % 8 == 0 and vdim % 8 == 0 and dim <= 256 and vdim <= 256
+            and os.environ.get("MEGATRON_AMD_NO_MFMA_MAPS", "0") != "1")
+
+
+def _map_split(batch, nblk):
+    return max(1, min((batch.max_context + 63) // 64, 1024 // max(nblk, 1), 64))
+
+
+def map_attention(q, pool, heads, kv_heads, maps, dim, vdim, scale, softcap, batch):
+    """-> fp32 [T, heads * maps * vdim]: the result of every softmax map of every head"""
+    if _native_g(q):
+        if _map_mfma_ok(q, dim, vdim):
+            tiles = batch.row_tiles(heads // kv_heads, q.device)
+            nsplit = _map_split(batch, tiles.shape[0] * kv_heads * maps)
+            return _G.map_attention_mfma(q, _none(q.device), pool, int(heads), int(kv_heads), int(maps), int(dim),
+                                         int(vdim), float(scale), float(softcap), tiles, batch.cu_tokens,
+                                         batch.start_pos, batch.block_tables, int(batch.block_size), int(nsplit))
+        return _G.map_attention(q, pool, int(heads), int(kv_heads), int(maps), int(dim), int(vdim), float(scale),
+                                float(softcap), batch.tok_req, batch.tok_pos, batch.block_tables,
+                                int(batch.block_size))
+    return ref.map_attention(q, pool, heads, kv_heads, maps, dim, vdim, scale, softcap, batch)
+
+
+def softcap_gated_attention(q, gate, pool, heads, kv_heads, dim, vdim, scale, softcap, batch):
+    """Causal grouped-query attention with capped scores whose concatenated heads
+    are multiplied by sigmoid(gate [T, heads*vdim]) -> [T, heads*vdim] in q's dtype."""
+    if _native_g(q):
+        if _map_mfma_ok(q, dim, vdim):
+            # matrix-core kernel, gate applied when the result leaves the accumulators
+            tiles = batch.row_tiles(heads // kv_heads, q.device)
+            nsplit = _map_split(batch, tiles.shape[0] * kv_heads)
+            return _G.map_attention_mfma(q, gate, pool, int(heads), int(kv_heads), 1, int(dim), int(vdim),
+                                         float(scale), float(softcap), tiles, batch.cu_tokens, batch.start_pos,
+                                         batch.block_tables, int(batch.block_size), int(nsplit))
+        A = map_attention(q, pool, heads, kv_heads, 1, dim, vdim, scale, softcap, batch)
+        return _G.gate_finish(A, gate, q.dtype == torch.bfloat16)
+    A = ref.map_attention(q, pool, heads, kv_heads, 1, dim, vdim, scale, softcap, batch)
+    return ref.gate_finish(A, gate, q.dtype)
+
+
+def differential_attention(q, gate, lam, diff, eps, pool, heads, kv_heads, dim, vdim, scale, batch):
+    """Two softmax maps a head over the same values: o = a1 - lam a2, unit-normed
+    per head, times (1 - diff) sigmoid(gate [T, heads]) -> [T, heads*vdim] in q's dtype."""
+    A = map_attention(q, pool, heads, kv_heads, 2, dim, vdim, scale, 0.0, batch)
+    if _native_g(q):
+        return _G.differential_finish(A, gate, lam, float(diff), float(eps), int(heads), int(vdim),
+                                      q.dtype == torch.bfloat16)
+    return ref.differential_finish(A, gate, lam, diff, eps, heads, vdim, q.dtype)
+
+
+def relu2(z, out_dtype):
+    if _native_g(z):
+        return _G.relu2(z)
+    return ref.relu2(z, out_dtype)
+
+
+def expert_pairs_plain(h, ids, w_up, w_down):
+    """Experts without a gate matrix, down(relu(up x)^2), one (token, choice) pair a row."""
+    if _native_g(h):
+        return _G.expert_pairs_plain(h, ids, w_up, w_down)
+    return ref.expert_pairs_plain(h, ids, w_up, w_down)

@@ -420,10 +420,13 @@ def expert_pairs(h, ids, w_gate_up, w_down, limit, alpha, act="clamped"):
 def moe_router(h, w_router, experts, top, groups, keep, scale, bias=None, score="sigmoid"):
     """Router in one call: fp32 logits of all rows of w_router (+ bias; the rows
     beyond ``experts`` are returned raw), then moe_route (score "sigmoid") or
-    moe_route_softmax (score "softmax").  -> (ids, weights, extra [T, rows - experts])"""
+    moe_route_softmax (score "softmax") or moe_route_softmax_all (score
+    "softmax_all").  -> (ids, weights, extra [T, rows - experts])"""
     logits = F.linear(h.float(), w_router.float(), bias.float() if bias is not None else None)
     if score == "softmax":
         ids, weights = moe_route_softmax(logits[:, :experts], top)
+    elif score == "softmax_all":
+        ids, weights = moe_route_softmax_all(logits[:, :experts], top)
     else:
         ids, weights = moe_route(logits, experts, top, groups, keep, scale)
     return ids, weights, logits[:, experts:].contiguous()
@@ -550,3 +553,178 @@ def moe_route_softmax(logits, top):
     logits only.  -> (ids [T, top] int32, weights [T, top] fp32)."""
     val, idx = logits.float().topk(top, dim=-1)
     return idx.to(torch.int32), torch.softmax(val, dim=-1)
+
+
+# ---------------------------------------------------------------------------
+# norms on both sides of a sublayer, restart of a repeated block of layers,
+# rotation in pairs or halves with wavelength-dependent frequency scaling and an
+# optional unit norm, attention with several softmax maps per head over shared
+# values (capped scores, gated or differential finish), squared ReLU, routing by
+# the softmax over all experts, experts without a gate matrix
+# ---------------------------------------------------------------------------
+
+
+def sandwich_norm_add(x, y, w_post, w_pre, eps, out_dtype, copy_to=None):
+    """x fp32 [T, W] <- x + y / sqrt(mean(y^2) + eps) * w_post in place (skipped
+    when ``y`` is None).  ``copy_to`` ([T, W] view, any row stride) receives the
+    new x in its own dtype.  Returns x / sqrt(mean(x^2) + eps) * w_pre in
+    ``out_dtype`` (None when ``w_pre`` is None)."""
+    if y is not None:
+        yf = y.float()
+        x.add_(yf * torch.rsqrt((yf * yf).mean(-1, keepdim=True) + eps) * w_post.float())
+    if copy_to is not None:
+        copy_to.copy_(x)
+    if w_pre is None:
+        return None
+    return (x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * w_pre.float()).to(out_dtype)
+
+
+def restart_norm(y, bias, w_pre, eps, out_dtype):
+    """A fresh fp32 residual x = y + bias (bias [W]) and its normed copy
+    x / sqrt(mean(x^2) + eps) * w_pre in ``out_dtype``.  -> (x, h)"""
+    x = y.float() + bias.float()
+    return x, (x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * w_pre.float()).to(out_dtype)
+
+
+def scaled_freqs(dims, base, scaling=None, device=None):
+    """f_i = base^(-2i/dims), i < dims/2, in float64; with ``scaling`` (factor,
+    low, high, original): a wavelength 2 pi / f below original/high keeps f, one
+    above original/low uses f / factor, and between them
+    s = (original / wavelength - low) / (high - low) blends (1 - s) f / factor + s f.
+    Rounded once to fp32."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims)
+    if scaling:
+        factor, low, high = float(scaling["factor"]), float(scaling["low"]), float(scaling["high"])
+        orig = float(scaling["original"])
+        wl = 2.0 * math.pi / f
+        s = (orig / wl - low) / (high - low)
+        mid = (1.0 - s) * f / factor + s * f
+        f = torch.where(wl < orig / high, f, torch.where(wl > orig / low, f / factor, mid))
+    return f.to(torch.float32).to(device)
+
+
+ROT_LAYOUTS = {"pairs": 0, "halves": 1}
+
+
+def _rotate_layout(x, pos, freqs, layout):
+    """x [T, heads, d] fp32; "pairs": entries (2i, 2i+1), "halves": (i, i + n),
+    i < n = len(freqs), rotated by pos * f_i."""
+    n = freqs.numel()
+    if n == 0:
+        return x
+    if layout == "pairs":
+        return _rotate_pairs(x, pos, freqs)
+    ang = pos.float()[:, None, None] * freqs.float()[None, None, :]
+    c, s = torch.cos(ang), torch.sin(ang)
+    u, v = x[..., :n], x[..., n:2 * n]
+    out = x.clone()
+    out[..., :n] = u * c - v * s
+    out[..., n:2 * n] = v * c + u * s
+    return out
+
+
+def rope_norm_store(proj, q_heads, k_heads, dim, v_width, freqs, layout, unit_norm, eps, pool, batch):
+    """proj [T, q_heads*dim | k_heads*dim | v_width | ...] (columns beyond the
+    values are not read).  Every q and k head is rotated by the token's position
+    (``layout``: "pairs" or "halves", first 2 len(freqs) entries) and then, with
+    ``unit_norm``, divided by its root mean square.  Cache row <- [k | v];
+    returns q [T, q_heads*dim]."""
+    T = proj.shape[0]
+    D = dim
+    pf = proj.float()
+    q = pf[:, :q_heads * D].view(T, q_heads, D)
+    k = pf[:, q_heads * D:(q_heads + k_heads) * D].view(T, k_heads, D)
+    v = pf[:, (q_heads + k_heads) * D:(q_heads + k_heads) * D + v_width]
+    q = _rotate_layout(q, batch.tok_pos, freqs, layout)
+    k = _rotate_layout(k, batch.tok_pos, freqs, layout)
+    if unit_norm:
+        q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + eps)
+        k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + eps)
+    pool[batch.tok_row] = torch.cat([k.reshape(T, k_heads * D), v], dim=-1).to(pool.dtype)
+    return q.reshape(T, q_heads * D).to(proj.dtype)
+
+
+def map_attention(q, pool, heads, kv_heads, maps, dim, vdim, scale, softcap, batch):
+    """Causal softmax attention over the paged cache with ``maps`` softmax maps a
+    head.  q [T, heads*maps*dim], head-major then map; cache rows
+    [kv_heads*maps*dim keys | kv_heads*vdim values]: map m of query head h reads
+    key (h // rep, m) and the values of key/value head h // rep.
+        s = q . k * scale;  softcap > 0: s <- softcap tanh(s / softcap)
+    -> fp32 [T, heads*maps*vdim]."""
+    T = q.shape[0]
+    H, G, M, D, V = heads, kv_heads, maps, dim, vdim
+    rep = H // G
+    bs = batch.block_size
+    dev = q.device
+    out = torch.empty(T, H * M * V, dtype=torch.float32, device=dev)
+    hm = torch.arange(H * M, device=dev)
+    key_of = (hm // (rep * M)) * M + hm % M
+    val_of = hm // (rep * M)
+    for r, a, b, start, slot in _spans(batch):
+        n = b - a
+        L = start + n
+        table = torch.as_tensor(batch.host_tables[r], dtype=torch.long, device=dev)
+        kv = pool[_rows_of(table, L, bs, dev)].float()
+        keys = kv[:, :G * M * D].view(-1, G * M, D)
+        vals = kv[:, G * M * D:].view(-1, G, V)
+        qi = torch.arange(start, L, device=dev)
+        j = torch.arange(L, device=dev)
+        ok = j[None, :] <= qi[:, None]
+        qq = q[a:b].float().view(n, H * M, D)
+        s = torch.einsum("nhd,lhd->nhl", qq, keys[:, key_of]) * scale
+        if softcap > 0:
+            s = softcap * torch.tanh(s / softcap)
+        s = s.masked_fill(~ok[:, None, :], float("-inf"))
+        p = torch.softmax(s, dim=-1)
+        out[a:b] = torch.einsum("nhl,lhv->nhv", p, vals[:, val_of]).reshape(n, H * M * V)
+    return out
+
+
+def gate_finish(A, gate, out_dtype):
+    """A fp32 [T, N] * sigmoid(gate [T, N]) -> out_dtype"""
+    return (A * torch.sigmoid(gate.float())).to(out_dtype)
+
+
+def differential_finish(A, gate, lam, diff, eps, heads, vdim, out_dtype):
+    """A fp32 [T, heads*2*vdim] = the two maps' results (a1, a2) per head;
+    o = a1 - lam a2, o <- o / sqrt(mean(o^2) + eps) * (1 - diff), times
+    sigmoid(gate[t, head]).  -> [T, heads*vdim] in out_dtype."""
+    T = A.shape[0]
+    a = A.view(T, heads, 2, vdim)
+    o = a[:, :, 0] - lam.float().reshape(()) * a[:, :, 1]
+    o = o * torch.rsqrt((o * o).mean(-1, keepdim=True) + eps) * (1.0 - diff)
+    o = o * torch.sigmoid(gate.float())[:, :, None]
+    return o.reshape(T, heads * vdim).to(out_dtype)
+
+
+def relu2(z, out_dtype):
+    """max(z, 0)^2"""
+    r = torch.relu(z.float())
+    return (r * r).to(out_dtype)
+
+
+def gelu_glu(gu, out_dtype):
+    """gu [N, 2F] = [gate | up]: y = gelu_tanh(gate) up."""
+    F_ = gu.shape[1] // 2
+    return (gelu_tanh(gu[:, :F_], torch.float32) * gu[:, F_:].float()).to(out_dtype)
+
+
+def moe_route_softmax_all(logits, top):
+    """Scores = softmax over ALL experts; the ``top`` largest are chosen and
+    keep their own scores as weights (they do not sum to one).
+    -> (ids [T, top] int32, weights [T, top] fp32)."""
+    val, idx = torch.softmax(logits.float(), dim=-1).topk(top, dim=-1)
+    return idx.to(torch.int32), val
+
+
+def expert_pairs_plain(h, ids, w_up, w_down):
+    """Every (token, choice) pair through its expert without a gate matrix,
+    down(relu(up x)^2); rows in pair order (token-major)."""
+    T, K = ids.shape
+    out = torch.empty(T * K, h.shape[1], dtype=h.dtype, device=h.device)
+    for t in range(T):
+        for k in range(K):
+            e = int(ids[t, k])
+            out[t * K + k] = F.linear(relu2(F.linear(h[t:t + 1], w_up[e]), h.dtype), w_down[e])[0]
+    return out

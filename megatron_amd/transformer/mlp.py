@@ -91,3 +91,21 @@ class GeluMLP(nn.Module):
         from megatron_amd.ops import ragged as R
 
         return F.linear(R.gelu_tanh(F.linear(h, self.w_up), h.dtype), self.w_down)
+
+
+class GeluGLUMLP(nn.Module):
+    """Dense gated feed-forward without biases, down(gelu_tanh(gate h) * (up h));
+    [gate; up] is one matrix (ops.ragged.glu, kind "gelu_tanh").  Plain replicated
+    weights (serving path)."""
+
+    def __init__(self, hidden: int, ffn: int, dtype=torch.bfloat16):
+        super().__init__()
+        self.w_gate_up = nn.Parameter(torch.zeros(2 * ffn, hidden, dtype=dtype))
+        self.w_down = nn.Parameter(torch.zeros(hidden, ffn, dtype=dtype))
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        import torch.nn.functional as F
+
+        from megatron_amd.ops import ragged as R
+
+        return F.linear(R.glu(F.linear(h, self.w_gate_up), "gelu_tanh", 0.0, 0.0, h.dtype), self.w_down)
