@@ -1,4 +1,5 @@
-// Routed GLU experts (clamped, kind 0, or SiLU, kind 1) for steps with few (token, choice) pairs
+// Routed GLU experts (clamped, kind 0, SiLU, kind 1, tanh-GELU, kind 2) and experts without a gate
+// matrix (squared ReLU) for steps with few (token, choice) pairs
 // (decoding): every pair reads its expert's matrices directly, no sorting, no
 // host read.  Two kernels:
 //   y[pair, f]   = act(W_gate[e][f] . x, W_up[e][f] . x)     grid (pair, tiles of rows f)
@@ -62,8 +63,10 @@ __global__ __launch_bounds__(256) void expert_gate_up_kernel(
         g = fminf(g, limit);
         u = fminf(fmaxf(u, -limit), limit);
         stf(y + (long)pair * F + f, g * sigmoidf_(alpha * g) * (u + 1.f));
-      } else {
+      } else if (kind == 1) {
         stf(y + (long)pair * F + f, g * sigmoidf_(g) * u);
+      } else {
+        stf(y + (long)pair * F + f, 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u);
       }
     }
   }
@@ -96,10 +99,72 @@ __global__ __launch_bounds__(256) void expert_down_kernel(const T* __restrict__ 
   }
 }
 
+// experts WITHOUT a gate matrix: y[pair, f] = max(W_up[e][f] . x, 0)^2
+template <typename T>
+__global__ __launch_bounds__(256) void expert_up_relu2_kernel(
+    const T* __restrict__ h, const int* __restrict__ ids, const T* __restrict__ wu, T* __restrict__ y, int K,
+    int W, int F) {
+  extern __shared__ float xs[];                  // the token's input, fp32
+  const int pair = blockIdx.x, t = pair / K;
+  const long e = ids[pair];
+  for (int i = threadIdx.x; i < W; i += 256) xs[i] = ldf(h + (long)t * W + i);
+  __syncthreads();
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const T* base = wu + e * (long)F * W;
+  for (int fi = wave; fi < EP_ROWS; fi += 4) {
+    const int f = blockIdx.y * EP_ROWS + fi;
+    if (f >= F) break;
+    const T* ur = base + (long)f * W;
+    float au = 0.f;
+    for (int d = lane * 8; d < W; d += WAVE * 8) {
+      float b[8];
+      load8<T>(ur + d, b);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) au += b[i] * xs[d + i];
+    }
+    au = wave_reduce_sum(au);
+    if (lane == 0) {
+      // the product's result takes the storage type's rounding, as a GEMM's output would
+      float u = au;
+      if (sizeof(T) == 2) u = sbf2f(f2sbf(u));
+      u = fmaxf(u, 0.f);
+      stf(y + (long)pair * F + f, u * u);
+    }
+  }
+}
+
+// h [T, W], ids [T, K], w_up [E, F, W], w_down [E, W, F] -> rows [T * K, W] in pair order (token-major)
+torch::Tensor expert_pairs_plain(torch::Tensor h, torch::Tensor ids, torch::Tensor wu, torch::Tensor wd) {
+  TORCH_CHECK(h.is_cuda() && h.dim() == 2 && h.is_contiguous());
+  check_i32(ids, "ids");
+  TORCH_CHECK(wu.is_contiguous() && wu.dim() == 3 && wd.is_contiguous() && wd.dim() == 3);
+  TORCH_CHECK(wu.scalar_type() == h.scalar_type() && wd.scalar_type() == h.scalar_type());
+  const int T_ = h.size(0), W = h.size(1), E = wu.size(0), F = wu.size(1);
+  TORCH_CHECK(ids.dim() == 2 && ids.size(0) == T_);
+  const int K = ids.size(1);
+  TORCH_CHECK(wu.size(2) == W && wd.size(0) == E && wd.size(1) == W && wd.size(2) == F);
+  TORCH_CHECK(W % 8 == 0 && F % 8 == 0, "pair kernels take widths that are multiples of 8");
+  TORCH_CHECK((size_t)std::max(W, F) * sizeof(float) <= 60 * 1024, "input vector above the LDS staging size");
+  const int N = T_ * K;
+  auto out = torch::empty({N, W}, h.options());
+  if (N == 0) return out;
+  auto y = torch::empty({N, F}, h.options());
+  auto stream = at::cuda::getCurrentHIPStream();
+  RAGGED_DISPATCH(h, {
+    hipLaunchKernelGGL((expert_up_relu2_kernel<T>), dim3(N, (F + EP_ROWS - 1) / EP_ROWS), dim3(256),
+        (size_t)W * sizeof(float), stream, (const T*)h.data_ptr(), ids.data_ptr<int>(), (const T*)wu.data_ptr(),
+        (T*)y.data_ptr(), K, W, F);
+    hipLaunchKernelGGL((expert_down_kernel<T>), dim3(N, (W + EP_ROWS - 1) / EP_ROWS), dim3(256),
+        (size_t)F * sizeof(float), stream, (const T*)y.data_ptr(), ids.data_ptr<int>(), (const T*)wd.data_ptr(),
+        (T*)out.data_ptr(), W, F);
+  });
+  return out;
+}
+
 // h [T, W], ids [T, K] -> rows [T * K, W] in pair order (token-major)
 torch::Tensor expert_pairs(torch::Tensor h, torch::Tensor ids, torch::Tensor wgu, torch::Tensor wd, double limit,
                            double alpha, int64_t kind) {
-  TORCH_CHECK(kind == 0 || kind == 1, "GLU kind: 0 clamped, 1 SiLU");
+  TORCH_CHECK(kind >= 0 && kind <= 2, "GLU kind: 0 clamped, 1 SiLU, 2 tanh-GELU");
   TORCH_CHECK(h.is_cuda() && h.dim() == 2 && h.is_contiguous());
   check_i32(ids, "ids");
   TORCH_CHECK(wgu.is_contiguous() && wgu.dim() == 3 && wd.is_contiguous() && wd.dim() == 3);

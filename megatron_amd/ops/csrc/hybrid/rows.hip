@@ -180,7 +180,8 @@ std::vector<torch::Tensor> moe_route(torch::Tensor logits, int64_t E, int64_t to
 // router in one kernel: logits = W_r h (+ bias) in fp32 (W_r fp32, h from its
 // storage type), then either sigmoid scores, group-limited top-k and weights =
 // chosen scores / their sum * scale (score 0), or the largest logits and
-// weights = softmax over the chosen logits (score 1); rows beyond the experts
+// weights = softmax over the chosen logits (score 1) or their softmax over ALL
+// experts (score 2: the weights do not sum to one); rows beyond the experts
 // (a shared expert's gate vector) are returned as raw logits.
 // One workgroup per token: its eight waves take the rows of W_r in turn (16 B
 // loads, four partial sums), one thread selects from the scores in LDS.
@@ -258,6 +259,18 @@ __global__ __launch_bounds__(RF_THREADS) void moe_router_kernel(
     if (best >= 0) sc[best] = -INFINITY;          // taken
     sum += cs[n];
   }
+  if (score == 2) {                               // softmax over all experts; cs[0] is the largest logit
+    const float top0 = cs[0];
+    sum = 0.f;
+    for (int n = 0; n < top; ++n) sum += expf(cs[n] - top0);
+    for (int e = 0; e < E; ++e)                   // the chosen entries of sc were overwritten with -inf
+      if (sc[e] != -INFINITY) sum += expf(sc[e] - top0);
+    for (int n = 0; n < top; ++n) {
+      ids[t * top + n] = chosen[n];
+      wts[t * top + n] = expf(cs[n] - top0) / sum;
+    }
+    return;
+  }
   if (score != 0) {                               // softmax over the chosen logits; cs[0] is the largest
     sum = 0.f;
     const float top0 = cs[0];
@@ -286,7 +299,8 @@ std::vector<torch::Tensor> moe_router(torch::Tensor h, torch::Tensor wr, torch::
     check_f32(bias, "router bias");
     TORCH_CHECK(bias.numel() == wr.size(0), "one bias per router row");
   }
-  TORCH_CHECK(score == 0 || (score == 1 && groups == 1), "score: 0 sigmoid (groups allowed), 1 softmax over the chosen");
+  TORCH_CHECK(score == 0 || ((score == 1 || score == 2) && groups == 1),
+              "score: 0 sigmoid (groups allowed), 1 softmax over the chosen, 2 softmax over all experts");
   const int T_ = h.size(0), W = h.size(1), rows = wr.size(0);
   TORCH_CHECK(wr.dim() == 2 && wr.size(1) == W && E >= 1 && E <= rows && rows <= RF_MAX_ROWS);
   TORCH_CHECK(top >= 1 && top <= RT_MAX_TOP && top <= E, "experts chosen per token");
@@ -308,6 +322,7 @@ std::vector<torch::Tensor> moe_router(torch::Tensor h, torch::Tensor wr, torch::
 // ---------------------------------------------------------------------------
 // kind 0: y = g sigmoid(alpha g) (u + 1),  g = min(gate, limit), u = clamp(up, -limit, limit)
 // kind 1: y = gate sigmoid(gate) up
+// kind 2: y = gelu_tanh(gate) up,  gelu_tanh(z) = 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void clamped_glu_kernel(const T* __restrict__ gu, long stride, T* __restrict__ y, long N, int F,
@@ -321,14 +336,16 @@ __global__ void clamped_glu_kernel(const T* __restrict__ gu, long stride, T* __r
       g = fminf(g, limit);
       u = fminf(fmaxf(u, -limit), limit);
       stf(y + i, g * sigmoidf_(alpha * g) * (u + 1.f));
-    } else {
+    } else if (kind == 1) {
       stf(y + i, g * sigmoidf_(g) * u);
+    } else {
+      stf(y + i, 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u);
     }
   }
 }
 
 torch::Tensor clamped_glu(torch::Tensor gu, double limit, double alpha, int64_t kind) {
-  TORCH_CHECK(kind == 0 || kind == 1, "GLU kind: 0 clamped, 1 SiLU");
+  TORCH_CHECK(kind >= 0 && kind <= 2, "GLU kind: 0 clamped, 1 SiLU, 2 tanh-GELU");
   TORCH_CHECK(gu.is_cuda() && gu.dim() == 2 && gu.stride(1) == 1 && gu.size(1) % 2 == 0);
   const long N = gu.size(0);
   const int F = gu.size(1) / 2;

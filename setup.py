@@ -62,6 +62,19 @@ TALKING_SRC = [
     "megatron_amd/ops/csrc/ragged/recurrent.hip",
 ]
 
+# the extension of the models with norms on both sides of a sublayer, gated softcap attention
+# and differential attention; it carries the row and expert kernels it shares with the hybrid
+# extension through their sources
+GATED_SRC = [
+    "megatron_amd/ops/csrc/gated/bindings.cpp",
+    "megatron_amd/ops/csrc/gated/sandwich_norm.hip",
+    "megatron_amd/ops/csrc/gated/rope_store.hip",
+    "megatron_amd/ops/csrc/gated/map_attention.hip",
+    "megatron_amd/ops/csrc/gated/map_attention_mfma.hip",
+    "megatron_amd/ops/csrc/hybrid/rows.hip",
+    "megatron_amd/ops/csrc/hybrid/experts.hip",
+]
+
 # MEGATRON_AMD_ONLY_EXT=ragged builds just the serving kernels of the
 # ragged-batch models (what a fresh checkout compiles on first use); "hybrid"
 # likewise for the models built on the hybrid kernels
@@ -94,6 +107,12 @@ EXTS = {
         CUDAExtension(
             name="megatron_amd.ops._talking_ops",
             sources=TALKING_SRC,
+            extra_compile_args={"cxx": ["-O3", "-std=c++17"], "nvcc": HIPCC_FLAGS},
+        ),
+    "gated": lambda:
+        CUDAExtension(
+            name="megatron_amd.ops._gated_ops",
+            sources=GATED_SRC,
             extra_compile_args={"cxx": ["-O3", "-std=c++17"], "nvcc": HIPCC_FLAGS},
         ),
     "data": lambda:
