@@ -86,11 +86,15 @@ def parse_args():
     p.add_argument("--serve", action="store_true",
                    help="instead of the training step: prefill/decode throughput of the ragged-batch "
                         "Bezutar design beside GPT with multi-latent attention at equal sizes")
-    p.add_argument("--serve-design", default="bezutar", choices=["bezutar", "bezurax", "tilarax"],
+    p.add_argument("--serve-design", default="bezutar", choices=["bezutar", "bezurax", "tilarax", "lomazen"],
                    help="bezurax: also measure the Bezurax design (pooled-window attention beside a delta-rule "
                         "memory, routed experts) at the same sizes, before the patterns of --serve-patterns; "
                         "tilarax: likewise the Tilarax design (mLSTM and chunked talking-heads attention layers, "
-                        "post-sublayer norms with a depth-weighted residual history)")
+                        "post-sublayer norms with a depth-weighted residual history); lomazen: the Lomazen design "
+                        "(gated capped attention and differential attention, norms on both sides of a sublayer, a "
+                        "repeated block of layers) beside Tilarax with attention layers only, nothing else")
+    p.add_argument("--serve-models", default="lomazen,tilarax",
+                   help="with --serve-design lomazen: which of the two models to run (one of them for a profile)")
     p.add_argument("--serve-sizes", default="1b,7b-layers")
     p.add_argument("--serve-patterns", default="AMGA,A",
                    help="layer patterns of the new design: A latent attention, M mLSTM, G minGRU")

@@ -18,6 +18,13 @@ feed-forward size, both through the same ragged engine path.
 with chunked talking-heads attention layers, post-sublayer norms with a
 depth-weighted residual history, dense and routed feed-forwards in turn) next
 to the same Bezutar pattern.
+
+``--serve-design lomazen`` measures the Lomazen design (gated capped attention
+and differential attention layers with norms on both sides of every sublayer,
+a block of layers that runs twice, dense GELU-GLU and routed squared-ReLU
+feed-forwards in turn) next to Tilarax with attention layers only
+(``tilarax[aA]``: dense and routed feed-forwards in turn) at the same width,
+number of layer runs, head sizes and expert sizes.
 """
 
 from __future__ import annotations
@@ -90,7 +97,8 @@ T_SIZES = {
 }
 
 
-def tilarax_config(size):
+def tilarax_config(size, pattern="MA"):
+    """pattern, repeated over the depth: M mLSTM + dense, A attention + experts, a attention + dense"""
     s, x = SIZES[size], T_SIZES[size]
     rec = dict(type="mlstm", mixer=dict(heads=s["m_heads"], dim=s["m_dim"], vdim=s["m_vdim"], gate_cap=15.0),
                mlp=dict(kind="dense", ff=s["ff"]))
@@ -98,8 +106,39 @@ def tilarax_config(size):
                mixer=dict(heads=x["heads"], kv_heads=x["kv"], dim=x["dim"], vdim=x["dim"], scale=x["dim"] ** -0.5,
                           mask=dict(size=x["chunk"]), rot=dict(base=10000.0, dims=x["rot"]), v_mix=True),
                mlp=dict(kind="moe", expert=dict(ff=x["eff"]), router=dict(experts=x["experts"], top=x["top"])))
-    layers = [json.loads(json.dumps(att if i % 2 else rec)) for i in range(s["layers"])]
+    att_dense = dict(att, mlp=dict(kind="dense", ff=s["ff"]))
+    kinds = {"M": rec, "A": att, "a": att_dense}
+    layers = [json.loads(json.dumps(kinds[pattern[i % len(pattern)]])) for i in range(s["layers"])]
     return dict(architecture="Tilarax", vocab=s["vocab"], width=s["width"], norm=dict(eps=1e-6), layers=layers)
+
+
+# Lomazen at the same widths: gated attention layers (query heads x 128, a quarter as many kv heads,
+# capped scores, every head rotated with rescaled frequencies) with a dense feed-forward alternate
+# with differential attention layers (half as many heads, two maps of 128 each, values of 256, a
+# quarter of every map rotated) with 16 experts of which 4 are chosen; the middle layers run twice,
+# so that the number of layer runs equals the depth of the comparison
+L_SIZES = {
+    "1b": dict(layers=6, loop=(2, 4, 2)),
+    "7b-layers": dict(layers=3, loop=(1, 2, 2)),
+}
+
+
+def lomazen_config(size):
+    s, x, z = SIZES[size], T_SIZES[size], L_SIZES[size]
+    one = dict(type="attention",
+               mixer=dict(heads=x["heads"], kv_heads=x["kv"], dim=x["dim"], vdim=x["dim"], scale=x["dim"] ** -0.5,
+                          softcap=30.0, rot=dict(base=1000000.0, dims=x["dim"],
+                                                 scaling=dict(factor=8.0, low=1.0, high=4.0, original=1024))),
+               mlp=dict(kind="dense", ff=s["ff"]))
+    two = dict(type="attention_2",
+               mixer=dict(heads=x["heads"] // 2, kv_heads=max(1, x["kv"] // 2), dim=x["dim"], vdim=2 * x["dim"],
+                          scale=x["dim"] ** -0.5, diff=0.5, rot=dict(base=10000.0, dims=x["dim"] // 4)),
+               mlp=dict(kind="moe", expert=dict(ff=x["eff"]), router=dict(experts=x["experts"], top=x["top"])))
+    layers = [json.loads(json.dumps(two if i % 2 else one)) for i in range(z["layers"])]
+    a, b, t = z["loop"]
+    assert a + (b - a) * t + (z["layers"] - b) == s["layers"], "layer runs equal the comparison's depth"
+    return dict(architecture="Lomazen", vocab=s["vocab"], width=s["width"], norm=dict(eps=1e-6), logit_scale=1.0,
+                loop=dict(start=a, stop=b, times=t), layers=layers)
 
 
 def _random_init(model, seed=0):
@@ -152,14 +191,24 @@ def run_bezurax(size, batch, isl, osl, device):
     return _run_ragged(model, "bezurax", size, batch, isl, osl, device)
 
 
-def run_tilarax(size, batch, isl, osl, device):
+def run_tilarax(size, batch, isl, osl, device, pattern="MA"):
     from megatron_amd.models.tilarax import TilaraxConfig, TilaraxModel
 
-    cfg = TilaraxConfig.from_dict(tilarax_config(size), dtype=torch.bfloat16)
+    cfg = TilaraxConfig.from_dict(tilarax_config(size, pattern), dtype=torch.bfloat16)
     with torch.device(device):
         model = TilaraxModel(cfg).eval()
     _random_init(model)
-    return _run_ragged(model, "tilarax", size, batch, isl, osl, device)
+    return _run_ragged(model, "tilarax" if pattern == "MA" else f"tilarax[{pattern}]", size, batch, isl, osl, device)
+
+
+def run_lomazen(size, batch, isl, osl, device):
+    from megatron_amd.models.lomazen import LomazenConfig, LomazenModel
+
+    cfg = LomazenConfig.from_dict(lomazen_config(size), dtype=torch.bfloat16)
+    with torch.device(device):
+        model = LomazenModel(cfg).eval()
+    _random_init(model)
+    return _run_ragged(model, "lomazen", size, batch, isl, osl, device)
 
 
 def _run_ragged(model, label, size, batch, isl, osl, device):
@@ -257,6 +306,18 @@ def main(args) -> None:
             r.update(batch=args.serve_batch, isl=args.serve_isl, osl=args.serve_osl, dtype="bf16", data="synthetic")
             print(json.dumps(r), flush=True)
             torch.cuda.empty_cache()
+        if design == "lomazen":
+            # the new design, then the closest existing one (attention layers only); no Bezutar patterns
+            which = getattr(args, "serve_models", "lomazen,tilarax").split(",")
+            for name in which:
+                if name == "lomazen":
+                    r = run_lomazen(size, args.serve_batch, args.serve_isl, args.serve_osl, device)
+                else:
+                    r = run_tilarax(size, args.serve_batch, args.serve_isl, args.serve_osl, device, "aA")
+                r.update(batch=args.serve_batch, isl=args.serve_isl, osl=args.serve_osl, dtype="bf16", data="synthetic")
+                print(json.dumps(r), flush=True)
+                torch.cuda.empty_cache()
+            continue
         for pattern in [p for p in args.serve_patterns.split(",") if p and p != "none"]:
             r = run_bezutar(size, pattern, args.serve_batch, args.serve_isl, args.serve_osl, device)
             r.update(batch=args.serve_batch, isl=args.serve_isl, osl=args.serve_osl, dtype="bf16", data="synthetic")

@@ -83,19 +83,30 @@ __global__ __launch_bounds__(256) void expert_down_kernel(const T* __restrict__ 
   __syncthreads();
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const T* base = wd + e * (long)W * F;
-  for (int wi = wave; wi < EP_ROWS; wi += 4) {
-    const int w = blockIdx.y * EP_ROWS + wi;
-    if (w >= W) break;
-    const T* row = base + (long)w * F;
-    float acc = 0.f;
+  // two rows in flight a wave: rows wi and wi + 4 of the workgroup's EP_ROWS
+  for (int wi = wave; wi < EP_ROWS; wi += 8) {
+    const int w0 = blockIdx.y * EP_ROWS + wi, w1 = w0 + 4;
+    if (w0 >= W) break;
+    const bool two = w1 < W && wi + 4 < EP_ROWS;
+    const T* r0 = base + (long)w0 * F;
+    const T* r1 = base + (long)(two ? w1 : w0) * F;
+    float a0 = 0.f, a1 = 0.f;
     for (int d = lane * 8; d < F; d += WAVE * 8) {
-      float a[8];
-      load8<T>(row + d, a);
+      float b0[8], b1[8];
+      load8<T>(r0 + d, b0);
+      load8<T>(r1 + d, b1);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc += a[i] * ys[d + i];
+      for (int i = 0; i < 8; ++i) {
+        a0 += b0[i] * ys[d + i];
+        a1 += b1[i] * ys[d + i];
+      }
     }
-    acc = wave_reduce_sum(acc);
-    if (lane == 0) stf(out + (long)pair * W + w, acc);
+    a0 = wave_reduce_sum(a0);
+    a1 = wave_reduce_sum(a1);
+    if (lane == 0) {
+      stf(out + (long)pair * W + w0, a0);
+      if (two) stf(out + (long)pair * W + w1, a1);
+    }
   }
 }
 
@@ -111,24 +122,34 @@ __global__ __launch_bounds__(256) void expert_up_relu2_kernel(
   __syncthreads();
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const T* base = wu + e * (long)F * W;
-  for (int fi = wave; fi < EP_ROWS; fi += 4) {
-    const int f = blockIdx.y * EP_ROWS + fi;
-    if (f >= F) break;
-    const T* ur = base + (long)f * W;
-    float au = 0.f;
+  // two rows in flight a wave: rows fi and fi + 4 of the workgroup's EP_ROWS
+  for (int fi = wave; fi < EP_ROWS; fi += 8) {
+    const int f0 = blockIdx.y * EP_ROWS + fi, f1 = f0 + 4;
+    if (f0 >= F) break;
+    const bool two = f1 < F && fi + 4 < EP_ROWS;
+    const T* r0 = base + (long)f0 * W;
+    const T* r1 = base + (long)(two ? f1 : f0) * W;
+    float a0 = 0.f, a1 = 0.f;
     for (int d = lane * 8; d < W; d += WAVE * 8) {
-      float b[8];
-      load8<T>(ur + d, b);
+      float b0[8], b1[8];
+      load8<T>(r0 + d, b0);
+      load8<T>(r1 + d, b1);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) au += b[i] * xs[d + i];
+      for (int i = 0; i < 8; ++i) {
+        a0 += b0[i] * xs[d + i];
+        a1 += b1[i] * xs[d + i];
+      }
     }
-    au = wave_reduce_sum(au);
+    a0 = wave_reduce_sum(a0);
+    a1 = wave_reduce_sum(a1);
     if (lane == 0) {
       // the product's result takes the storage type's rounding, as a GEMM's output would
-      float u = au;
-      if (sizeof(T) == 2) u = sbf2f(f2sbf(u));
-      u = fmaxf(u, 0.f);
-      stf(y + (long)pair * F + f, u * u);
+      float u0 = a0, u1 = a1;
+      if (sizeof(T) == 2) { u0 = sbf2f(f2sbf(u0)); u1 = sbf2f(f2sbf(u1)); }
+      u0 = fmaxf(u0, 0.f);
+      u1 = fmaxf(u1, 0.f);
+      stf(y + (long)pair * F + f0, u0 * u0);
+      if (two) stf(y + (long)pair * F + f1, u1 * u1);
     }
   }
 }

@@ -319,47 +319,6 @@ std::vector<torch::Tensor> moe_router(torch::Tensor h, torch::Tensor wr, torch::
   return {ids, wts, extra};
 }
 
-// ---------------------------------------------------------------------------
-// kind 0: y = g sigmoid(alpha g) (u + 1),  g = min(gate, limit), u = clamp(up, -limit, limit)
-// kind 1: y = gate sigmoid(gate) up
-// kind 2: y = gelu_tanh(gate) up,  gelu_tanh(z) = 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
-// ---------------------------------------------------------------------------
-template <typename T>
-__global__ void clamped_glu_kernel(const T* __restrict__ gu, long stride, T* __restrict__ y, long N, int F,
-                                   float limit, float alpha, int kind) {
-  const long total = N * F;
-  for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
-    const long n = i / F;
-    const int f = (int)(i % F);
-    float g = ldf(gu + n * stride + f), u = ldf(gu + n * stride + F + f);
-    if (kind == 0) {
-      g = fminf(g, limit);
-      u = fminf(fmaxf(u, -limit), limit);
-      stf(y + i, g * sigmoidf_(alpha * g) * (u + 1.f));
-    } else if (kind == 1) {
-      stf(y + i, g * sigmoidf_(g) * u);
-    } else {
-      stf(y + i, 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u);
-    }
-  }
-}
-
-torch::Tensor clamped_glu(torch::Tensor gu, double limit, double alpha, int64_t kind) {
-  TORCH_CHECK(kind >= 0 && kind <= 2, "GLU kind: 0 clamped, 1 SiLU, 2 tanh-GELU");
-  TORCH_CHECK(gu.is_cuda() && gu.dim() == 2 && gu.stride(1) == 1 && gu.size(1) % 2 == 0);
-  const long N = gu.size(0);
-  const int F = gu.size(1) / 2;
-  auto y = torch::empty({N, F}, gu.options());
-  if (N == 0) return y;
-  auto stream = at::cuda::getCurrentHIPStream();
-  RAGGED_DISPATCH(gu, hipLaunchKernelGGL((clamped_glu_kernel<T>), dim3(grid_for(N * F, 256)), dim3(256), 0, stream,
-      (const T*)gu.data_ptr(), (long)gu.stride(0), (T*)y.data_ptr(), N, F, (float)limit, (float)alpha, (int)kind));
-  return y;
-}
-
-// ---------------------------------------------------------------------------
-// y[t] = sum_k w[t,k] down[inv[t,k]] + sigmoid(gate[t]) shared[t] + add[t]   (fp32)
-// ---------------------------------------------------------------------------
 template <typename T>
 __device__ __forceinline__ void load8_(const T* p, float* v);
 template <>
@@ -375,6 +334,87 @@ __device__ __forceinline__ void load8_<float>(const float* p, float* v) {
   for (int i = 0; i < 4; ++i) { v[i] = a[i]; v[4 + i] = b[i]; }
 }
 
+template <typename T>
+__device__ __forceinline__ void store8_(T* p, const float* v);
+template <>
+__device__ __forceinline__ void store8_<bf16>(bf16* p, const float* v) {
+  short8 x;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) x[i] = f2sbf(v[i]);
+  *reinterpret_cast<short8*>(p) = x;
+}
+template <>
+__device__ __forceinline__ void store8_<float>(float* p, const float* v) {
+  float4v* q = reinterpret_cast<float4v*>(p);
+  q[0] = float4v{v[0], v[1], v[2], v[3]};
+  q[1] = float4v{v[4], v[5], v[6], v[7]};
+}
+
+// ---------------------------------------------------------------------------
+// kind 0: y = g sigmoid(alpha g) (u + 1),  g = min(gate, limit), u = clamp(up, -limit, limit)
+// kind 1: y = gate sigmoid(gate) up
+// kind 2: y = gelu_tanh(gate) up,  gelu_tanh(z) = 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float glu_value_(float g, float u, float limit, float alpha, int kind) {
+  if (kind == 0) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g * sigmoidf_(alpha * g) * (u + 1.f);
+  }
+  if (kind == 1) return g * sigmoidf_(g) * u;
+  return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
+}
+
+// VEC: F and the row stride are multiples of 8 and the rows 16-byte aligned: 8 elements a thread and turn
+template <typename T, bool VEC>
+__global__ void clamped_glu_kernel(const T* __restrict__ gu, long stride, T* __restrict__ y, long N, int F,
+                                   float limit, float alpha, int kind) {
+  if (VEC) {
+    const int F8 = F / 8;
+    const long total = N * F8;
+    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+      const long n = i / F8;
+      const int f = (int)(i % F8) * 8;
+      float g[8], u[8];
+      load8_<T>(gu + n * stride + f, g);
+      load8_<T>(gu + n * stride + F + f, u);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) g[k] = glu_value_(g[k], u[k], limit, alpha, kind);
+      store8_<T>(y + n * F + f, g);
+    }
+    return;
+  }
+  const long total = N * F;
+  for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    const long n = i / F;
+    const int f = (int)(i % F);
+    stf(y + i, glu_value_(ldf(gu + n * stride + f), ldf(gu + n * stride + F + f), limit, alpha, kind));
+  }
+}
+
+torch::Tensor clamped_glu(torch::Tensor gu, double limit, double alpha, int64_t kind) {
+  TORCH_CHECK(kind >= 0 && kind <= 2, "GLU kind: 0 clamped, 1 SiLU, 2 tanh-GELU");
+  TORCH_CHECK(gu.is_cuda() && gu.dim() == 2 && gu.stride(1) == 1 && gu.size(1) % 2 == 0);
+  const long N = gu.size(0);
+  const int F = gu.size(1) / 2;
+  auto y = torch::empty({N, F}, gu.options());
+  if (N == 0) return y;
+  auto stream = at::cuda::getCurrentHIPStream();
+  const bool vec = F % 8 == 0 && gu.stride(0) % 8 == 0 &&
+                   reinterpret_cast<uintptr_t>(gu.data_ptr()) % 16 == 0;
+#define GLU_LAUNCH(VEC, COUNT)                                                                                   \
+  RAGGED_DISPATCH(gu, hipLaunchKernelGGL((clamped_glu_kernel<T, VEC>), dim3(grid_for(COUNT, 256)), dim3(256), 0, \
+      stream, (const T*)gu.data_ptr(), (long)gu.stride(0), (T*)y.data_ptr(), N, F, (float)limit, (float)alpha,   \
+      (int)kind))
+  if (vec) GLU_LAUNCH(true, N * (F / 8));
+  else GLU_LAUNCH(false, N * F);
+#undef GLU_LAUNCH
+  return y;
+}
+
+// ---------------------------------------------------------------------------
+// y[t] = sum_k w[t,k] down[inv[t,k]] + sigmoid(gate[t]) shared[t] + add[t]   (fp32)
+// ---------------------------------------------------------------------------
 // VEC: 8 elements per thread and pass with 16/32-byte accesses (W a multiple of 8), else one
 template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void moe_combine_kernel(
