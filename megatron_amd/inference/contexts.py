@@ -430,16 +430,17 @@ class RaggedBatch:
         """Work list of the matrix-core attention kernel: one entry
         (request, first row) per tile of ``rows_per_tile`` (token, head) rows,
         rows numbered token-major inside each request.  Cached per head count
-        (every attention layer of a step shares it)."""
+        and tile size (every attention layer of a step shares it)."""
         if self._tiles is None:
             self._tiles = {}
-        t = self._tiles.get(heads)
+        key = heads if rows_per_tile == 64 else (heads, rows_per_tile)
+        t = self._tiles.get(key)
         if t is None:
             work = []
             for r in range(self.num_requests):
                 rows = (self.host_cu[r + 1] - self.host_cu[r]) * heads
                 work.extend((r, row0) for row0 in range(0, rows, rows_per_tile))
-            t = self._tiles[heads] = torch.as_tensor(work, dtype=torch.int32).reshape(-1, 2).to(device)
+            t = self._tiles[key] = torch.as_tensor(work, dtype=torch.int32).reshape(-1, 2).to(device)
         return t
 
 

@@ -23,7 +23,7 @@ torch::Tensor map_attention(torch::Tensor q, torch::Tensor pool, int64_t H, int6
 torch::Tensor map_attention_mfma(torch::Tensor q, torch::Tensor gate, torch::Tensor pool, int64_t H, int64_t G,
                                  int64_t M, int64_t D, int64_t V, double scale, double cap, torch::Tensor tiles,
                                  torch::Tensor cu, torch::Tensor start_pos, torch::Tensor tables, int64_t bs,
-                                 int64_t nsplit);
+                                 int64_t nsplit, int64_t tile_rows);
 // hybrid/rows.hip, hybrid/experts.hip
 torch::Tensor embed_plain(torch::Tensor tokens, torch::Tensor embed);
 std::vector<torch::Tensor> residual_group_norm(torch::Tensor x, torch::Tensor y, torch::Tensor wa, torch::Tensor wb,

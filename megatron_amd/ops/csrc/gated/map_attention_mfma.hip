@@ -3,7 +3,9 @@
 //
 // Rows of the problem are (token, query head of the group) pairs of ONE request, ONE key/value
 // group g and ONE map m, i.e. the rep = H / G query rows (h, m), h in group g, that read key head
-// g * M + m and value head g; 64 per workgroup (16 per wave), numbered token-major.
+// g * M + m and value head g; 64 * RT per workgroup (RT tiles of 16 per wave), numbered token-major
+// (RT = 2 for steps with many rows: every staged tile, key fragment and gathered value fragment
+// then feeds twice the MFMAs; RT = 1 for steps with few rows).
 // blockIdx.z = g * M + m picks the key columns and the value columns of the cache row that are
 // staged, in tiles of 32 positions, as [key | value] in LDS.  A row at position p sees 0 .. p; the
 // tiles run to the workgroup's last token and the rest of a tile is masked per row.
@@ -15,9 +17,9 @@
 // The D fragment of S^T (lane (c, g4): kv = 4 g4 + r of two 16-key sub-tiles) is used directly as
 // the B fragment of the second product by numbering that MFMA's k slots (g4, j) -> kv = 4 g4 + j
 // (j < 4), 16 + 4 g4 + j - 4 (j >= 4); the A fragment gathers V in the same order.
-// Wave w computes S^T, the cap and the softmax of row tile w and publishes P^T (bf16, in
-// B-fragment order) and its rows' rescale factors in LDS; for the second product wave w owns the
-// value tiles n = w, w + 4, ... of ALL four row tiles.
+// Wave w computes S^T, the cap and the softmax of row tiles w RT .. w RT + RT - 1 and publishes P^T
+// (bf16, in B-fragment order) and its rows' rescale factors in LDS; for the second product wave w
+// owns the value tiles n = w, w + 4, ... of ALL 4 RT row tiles.
 //
 // Scores: s = q . k * scale; cap > 0: s <- cap * tanh(s / cap), tanh(x) = 1 - 2 / (exp(2x) + 1).
 // Result: with a gate (M = 1), out[t, h, :] = o * sigmoid(gate[t, h, :]) in bf16; without, the fp32
@@ -30,7 +32,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int MA_KT = 32;     // keys per tile
-constexpr int MA_ROWS = 64;   // rows per workgroup
+constexpr int MA_ROWS = 64;   // rows per workgroup and row tile of a wave
 constexpr float MA_NEG = -1e30f;
 constexpr int MA_MAX_SPLIT = 64;
 
@@ -39,7 +41,7 @@ __device__ __forceinline__ float fast_cap(float s, float cap, float two_inv_cap)
   return cap * (1.f - 2.f / (__expf(s * two_inv_cap) + 1.f));
 }
 
-template <int NKS, int NT>
+template <int NKS, int NT, int RT>
 __global__ __launch_bounds__(256) void map_attn_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ gate, long gstride, const bf16* __restrict__ pool,
     float scale, float cap, const int* __restrict__ tiles, const int* __restrict__ cu,
@@ -50,48 +52,57 @@ __global__ __launch_bounds__(256) void map_attn_mfma_kernel(
   constexpr int NTW = NT / 4;                    // value tiles per wave
   constexpr int KW = NKS * 32;                   // staged key columns (zero-padded)
   constexpr int ldk = KW + NT * 16 + 8;          // LDS row stride (bf16), padded against bank conflicts
-  extern __shared__ __align__(16) short lds[];   // [MA_KT][ldk] key|value tile | P^T [64][32] | factors [64]
+  constexpr int ROWS = MA_ROWS * RT, NRT = 4 * RT;   // rows and row tiles of the workgroup
+  extern __shared__ __align__(16) short lds[];   // [MA_KT][ldk] key|value tile | P^T [ROWS][32] | factors [ROWS]
   short* const p_lds = lds + MA_KT * ldk;
-  float* const f_lds = reinterpret_cast<float*>(p_lds + MA_ROWS * MA_KT);
+  float* const f_lds = reinterpret_cast<float*>(p_lds + ROWS * MA_KT);
   const int req = tiles[2 * blockIdx.x], row0 = tiles[2 * blockIdx.x + 1];
   const int kz = blockIdx.z, grp = kz / M, mp = kz % M, rep = H / G, HM = H * M;
   const int t0 = cu[req], n_rows = (cu[req + 1] - t0) * rep, start = start_pos[req];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g4 = lane >> 4;
   const int kcols = G * M * D, width = kcols + G * V;
 
-  // first product and softmax: wave w owns rows row0 + 16 w + (0..15), one per lane column c
-  const int my_row = row0 + wave * 16 + c;
-  const bool row_ok = my_row < n_rows;
-  const int my_tok = row_ok ? my_row / rep : 0;
-  const int my_qh = (grp * rep + (row_ok ? my_row % rep : 0)) * M + mp;
-  const int my_p = row_ok ? start + my_tok : -1;                    // the row's position
-  const float two_inv_cap = cap > 0.f ? 2.f / cap : 0.f;
-  const int last_row = min(row0 + MA_ROWS, n_rows) - 1;
-  const int p_max = start + last_row / rep;
-  int rt_pmax[4];                                                   // last position per row tile of 16
+  // first product and softmax: wave w owns rows row0 + 16 (w RT + j) + (0..15), one per lane column c
+  int my_tok[RT], my_qh[RT], my_p[RT];
+  bool row_ok[RT];
 #pragma unroll
-  for (int rt = 0; rt < 4; ++rt) {
+  for (int j = 0; j < RT; ++j) {
+    const int my_row = row0 + (wave * RT + j) * 16 + c;
+    row_ok[j] = my_row < n_rows;
+    my_tok[j] = row_ok[j] ? my_row / rep : 0;
+    my_qh[j] = (grp * rep + (row_ok[j] ? my_row % rep : 0)) * M + mp;
+    my_p[j] = row_ok[j] ? start + my_tok[j] : -1;                   // the row's position
+  }
+  const float two_inv_cap = cap > 0.f ? 2.f / cap : 0.f;
+  const int last_row = min(row0 + ROWS, n_rows) - 1;
+  const int p_max = start + last_row / rep;
+  int rt_pmax[NRT];                                                 // last position per row tile of 16
+#pragma unroll
+  for (int rt = 0; rt < NRT; ++rt) {
     const int first = row0 + rt * 16;
     rt_pmax[rt] = first < n_rows ? start + (min(first + 16, n_rows) - 1) / rep : -1;
   }
 
-  bf16x8 qb[NKS];
-  {
-    const bf16* qp = q + ((long)(t0 + my_tok) * HM + my_qh) * D;
+  bf16x8 qb[RT][NKS];
+#pragma unroll
+  for (int j = 0; j < RT; ++j) {
+    const bf16* qp = q + ((long)(t0 + my_tok[j]) * HM + my_qh[j]) * D;
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
       short8 v = short8{0, 0, 0, 0, 0, 0, 0, 0};
       const int d = ks * 32 + 8 * g4;
-      if (row_ok && d < D) v = *reinterpret_cast<const short8*>(qp + d);
-      qb[ks] = *reinterpret_cast<bf16x8*>(&v);
+      if (row_ok[j] && d < D) v = *reinterpret_cast<const short8*>(qp + d);
+      qb[j][ks] = *reinterpret_cast<bf16x8*>(&v);
     }
   }
-  f32x4 oacc[NTW][4];
+  f32x4 oacc[NTW][NRT];
 #pragma unroll
   for (int i = 0; i < NTW; ++i)
 #pragma unroll
-    for (int rt = 0; rt < 4; ++rt) oacc[i][rt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m = MA_NEG, l = 0.f;
+    for (int rt = 0; rt < NRT; ++rt) oacc[i][rt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m[RT], l[RT];
+#pragma unroll
+  for (int j = 0; j < RT; ++j) { m[j] = MA_NEG; l[j] = 0.f; }
 
   const int ntiles = p_max / MA_KT + 1;
   int tile_lo = 0, tile_hi = ntiles;
@@ -157,66 +168,77 @@ __global__ __launch_bounds__(256) void map_attn_mfma_kernel(
       if (s_row[k] >= 0) *reinterpret_cast<short8*>(lds + s_lds[k]) = stg[k];
     __syncthreads();
     if (tile + 1 < tile_hi) issue(tile + 1);
-    bool act[4];                                  // does row tile rt see anything of this key tile
+    bool act[NRT];                                // does row tile rt see anything of this key tile
 #pragma unroll
-    for (int rt = 0; rt < 4; ++rt) act[rt] = base <= rt_pmax[rt];
-    if (act[wave]) {                              // wave-uniform
-      f32x4 st[2], st2[2];
+    for (int rt = 0; rt < NRT; ++rt) act[rt] = base <= rt_pmax[rt];
+    bool mine = false;                            // does any row tile of this wave see the key tile (wave-uniform)
 #pragma unroll
-      for (int kvt = 0; kvt < 2; ++kvt) {
-        st[kvt] = f32x4{0.f, 0.f, 0.f, 0.f};
-        st2[kvt] = f32x4{0.f, 0.f, 0.f, 0.f};
-      }
+    for (int j = 0; j < RT; ++j) mine |= act[wave * RT + j];
+    if (mine) {
+      f32x4 st[RT][2], st2[RT][2];
+#pragma unroll
+      for (int j = 0; j < RT; ++j)
+#pragma unroll
+        for (int kvt = 0; kvt < 2; ++kvt) {
+          st[j][kvt] = f32x4{0.f, 0.f, 0.f, 0.f};
+          st2[j][kvt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
 #pragma unroll
         for (int kvt = 0; kvt < 2; ++kvt) {
           short8 tmp = *reinterpret_cast<const short8*>(lds + (kvt * 16 + c) * ldk + 8 * g4 + ks * 32);
-          if (ks & 1)
-            st2[kvt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<bf16x8*>(&tmp), qb[ks], st2[kvt],
-                                                               0, 0, 0);
-          else
-            st[kvt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<bf16x8*>(&tmp), qb[ks], st[kvt],
-                                                              0, 0, 0);
+          const bf16x8 kf = *reinterpret_cast<bf16x8*>(&tmp);
+#pragma unroll
+          for (int j = 0; j < RT; ++j) {
+            if (!act[wave * RT + j]) continue;
+            if (ks & 1) st2[j][kvt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qb[j][ks], st2[j][kvt], 0, 0, 0);
+            else st[j][kvt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qb[j][ks], st[j][kvt], 0, 0, 0);
+          }
         }
       }
-      st[0] += st2[0];
-      st[1] += st2[1];
-      float s[8];
-      bool ok[8];
-      float mx = MA_NEG;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int e = base + (i >> 2) * 16 + 4 * g4 + (i & 3);
-        ok[i] = e <= my_p;
-        s[i] = st[i >> 2][i & 3] * scale;
-        if (cap > 0.f) s[i] = fast_cap(s[i], cap, two_inv_cap);
-        if (ok[i]) mx = fmaxf(mx, s[i]);
-      }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m, mx);
-      const float corr = __expf(m - m_new);
-      m = m_new;
-      float psum = 0.f;
-      short8 pk;
+      for (int j = 0; j < RT; ++j) {
+        if (!act[wave * RT + j]) continue;
+        st[j][0] += st2[j][0];
+        st[j][1] += st2[j][1];
+        float sc[8];
+        bool ok[8];
+        float mx = MA_NEG;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float p = ok[i] ? __expf(s[i] - m_new) : 0.f;
-        psum += p;
-        pk[i] = f2sbf(p);
+        for (int i = 0; i < 8; ++i) {
+          const int e = base + (i >> 2) * 16 + 4 * g4 + (i & 3);
+          ok[i] = e <= my_p[j];
+          sc[i] = st[j][i >> 2][i & 3] * scale;
+          if (cap > 0.f) sc[i] = fast_cap(sc[i], cap, two_inv_cap);
+          if (ok[i]) mx = fmaxf(mx, sc[i]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m[j], mx);
+        const float corr = __expf(m[j] - m_new);
+        m[j] = m_new;
+        float psum = 0.f;
+        short8 pk;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float p = ok[i] ? __expf(sc[i] - m_new) : 0.f;
+          psum += p;
+          pk[i] = f2sbf(p);
+        }
+        l[j] = l[j] * corr + psum;
+        const int prow = (wave * RT + j) * 16 + c;
+        *reinterpret_cast<short8*>(p_lds + prow * MA_KT + g4 * 8) = pk;
+        if (g4 == 0) f_lds[prow] = corr;
       }
-      l = l * corr + psum;
-      *reinterpret_cast<short8*>(p_lds + (wave * 16 + c) * MA_KT + g4 * 8) = pk;
-      if (g4 == 0) f_lds[wave * 16 + c] = corr;
     }
     __syncthreads();
     {
-      bf16x8 pb[4];
-      float cr[4];
+      bf16x8 pb[NRT];
+      float cr[NRT];
       bool rescale = false;
 #pragma unroll
-      for (int rt = 0; rt < 4; ++rt) {
+      for (int rt = 0; rt < NRT; ++rt) {
         // a row tile that sees nothing of this key tile contributes P = 0 with factor 1
         short8 tmp = *reinterpret_cast<const short8*>(p_lds + (rt * 16 + c) * MA_KT + g4 * 8);
         const float f = f_lds[rt * 16 + c];
@@ -229,7 +251,7 @@ __global__ __launch_bounds__(256) void map_attn_mfma_kernel(
 #pragma unroll
         for (int i = 0; i < NTW; ++i)
 #pragma unroll
-          for (int rt = 0; rt < 4; ++rt) oacc[i][rt] *= cr[rt];
+          for (int rt = 0; rt < NRT; ++rt) oacc[i][rt] *= cr[rt];
       }
 #pragma unroll
       for (int i = 0; i < NTW; ++i) {
@@ -239,19 +261,24 @@ __global__ __launch_bounds__(256) void map_attn_mfma_kernel(
         for (int j = 0; j < 8; ++j) av[j] = vcol[((j >> 2) * 16 + 4 * g4 + (j & 3)) * ldk];
         const bf16x8 a = *reinterpret_cast<bf16x8*>(&av);
 #pragma unroll
-        for (int rt = 0; rt < 4; ++rt)
+        for (int rt = 0; rt < NRT; ++rt)
           if (act[rt]) oacc[i][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[rt], oacc[i][rt], 0, 0, 0);
       }
     }
     __syncthreads();
   }
-  l += __shfl_xor(l, 16, 64);
-  l += __shfl_xor(l, 32, 64);
+#pragma unroll
+  for (int j = 0; j < RT; ++j) {
+    l[j] += __shfl_xor(l[j], 16, 64);
+    l[j] += __shfl_xor(l[j], 32, 64);
+  }
   if (nsplit == 1) {
-    if (g4 == 0) f_lds[wave * 16 + c] = (row_ok && l > 0.f) ? 1.f / l : 0.f;
+#pragma unroll
+    for (int j = 0; j < RT; ++j)
+      if (g4 == 0) f_lds[(wave * RT + j) * 16 + c] = (row_ok[j] && l[j] > 0.f) ? 1.f / l[j] : 0.f;
     __syncthreads();
 #pragma unroll
-    for (int rt = 0; rt < 4; ++rt) {
+    for (int rt = 0; rt < NRT; ++rt) {
       const int row = row0 + rt * 16 + c;
       if (row < n_rows) {
         const float inv = f_lds[rt * 16 + c];
@@ -277,13 +304,15 @@ __global__ __launch_bounds__(256) void map_attn_mfma_kernel(
     }
   } else {
     const long rows_all = (long)Tn * HM;
-    if (g4 == 0 && row_ok) {
-      const long grow = (long)(t0 + my_tok) * HM + my_qh;
-      part_m[blockIdx.y * rows_all + grow] = m;
-      part_l[blockIdx.y * rows_all + grow] = l;
-    }
 #pragma unroll
-    for (int rt = 0; rt < 4; ++rt) {
+    for (int j = 0; j < RT; ++j)
+      if (g4 == 0 && row_ok[j]) {
+        const long grow = (long)(t0 + my_tok[j]) * HM + my_qh[j];
+        part_m[blockIdx.y * rows_all + grow] = m[j];
+        part_l[blockIdx.y * rows_all + grow] = l[j];
+      }
+#pragma unroll
+    for (int rt = 0; rt < NRT; ++rt) {
       const int row = row0 + rt * 16 + c;
       if (row < n_rows) {
         const long grow = (long)(t0 + row / rep) * HM + (grp * rep + row % rep) * M + mp;
@@ -335,7 +364,8 @@ __global__ void map_combine_kernel(const float* __restrict__ part_o, const float
 torch::Tensor map_attention_mfma(torch::Tensor q, torch::Tensor gate, torch::Tensor pool, int64_t H, int64_t G,
                                  int64_t M, int64_t D, int64_t V, double scale, double cap, torch::Tensor tiles,
                                  torch::Tensor cu, torch::Tensor start_pos, torch::Tensor tables, int64_t bs,
-                                 int64_t nsplit) {
+                                 int64_t nsplit, int64_t tile_rows) {
+  TORCH_CHECK(tile_rows == MA_ROWS || tile_rows == 2 * MA_ROWS, "rows a workgroup: 64 or 128 (what the tile list was made for)");
   TORCH_CHECK(q.is_cuda() && q.dim() == 2 && q.is_contiguous() && q.scalar_type() == at::kBFloat16 &&
               q.size(1) == H * M * D);
   TORCH_CHECK(pool.is_contiguous() && pool.dim() == 2 && pool.scalar_type() == at::kBFloat16 &&
@@ -374,18 +404,25 @@ torch::Tensor map_attention_mfma(torch::Tensor q, torch::Tensor gate, torch::Ten
   bf16* gatedp = has_gate ? (bf16*)out.data_ptr() : nullptr;
   const bf16* gatep = has_gate ? (const bf16*)gate.data_ptr() : nullptr;
   const dim3 grid(nblk, (unsigned)nsplit, (unsigned)(G * M));
-#define MA_MFMA(NKS, NT)                                                                                        \
-  hipLaunchKernelGGL((map_attn_mfma_kernel<NKS, NT>), grid, dim3(256),                                          \
-      ((size_t)MA_KT * (NKS * 32 + NT * 16 + 8) + MA_ROWS * MA_KT) * sizeof(short) + MA_ROWS * sizeof(float),   \
+#define MA_MFMA1(NKS, NT, RT)                                                                                   \
+  hipLaunchKernelGGL((map_attn_mfma_kernel<NKS, NT, RT>), grid, dim3(256),                                      \
+      ((size_t)MA_KT * (NKS * 32 + NT * 16 + 8) + MA_ROWS * RT * MA_KT) * sizeof(short) +                       \
+          MA_ROWS * RT * sizeof(float),                                                                         \
       stream, (const bf16*)q.data_ptr(), gatep, gstride, (const bf16*)pool.data_ptr(), (float)scale, (float)cap, \
       tiles.data_ptr<int>(), cu.data_ptr<int>(), start_pos.data_ptr<int>(), tables.data_ptr<int>(),             \
       (int)tables.size(1), (int)bs, outp, gatedp, pop, pmp, plp, (int)nsplit, T_, (int)H, (int)G, (int)M,       \
       (int)D, (int)V)
+#define MA_MFMA(NKS, NT)                        \
+  do {                                          \
+    if (tile_rows == MA_ROWS) MA_MFMA1(NKS, NT, 1); \
+    else MA_MFMA1(NKS, NT, 2);                  \
+  } while (0)
   if (nks <= 2 && nt <= 4) MA_MFMA(2, 4);
   else if (nks <= 2 && nt <= 8) MA_MFMA(2, 8);
   else if (nks <= 4 && nt <= 8) MA_MFMA(4, 8);
   else if (nks <= 4) MA_MFMA(4, 16);
   else MA_MFMA(8, 16);
+#undef MA_MFMA1
 #undef MA_MFMA
   if (nsplit > 1)
     hipLaunchKernelGGL(map_combine_kernel, dim3((unsigned)((long)T_ * H * M)), dim3(128), 0, stream, pop, pmp, plp,

@@ -5,21 +5,21 @@
 // ---------------------------------------------------------------------------
 // proj [T, QH*D | KH*D | VW | ...] (row stride given; later columns are not read)
 // -> q_out [T, QH*D], cache row [KH*D | VW].
-// Every head: entries of pair i < nrot rotated by pos * freqs[i]; layout 0 pairs
+// Every head: entries of pair i < nrot rotated by pos * freqs[i] (float64 product, fp32 sine and cosine); layout 0 pairs
 // (2i, 2i+1), layout 1 pairs (i, i + nrot); with unit: x / sqrt(mean(x^2) + eps).
 // Workgroup = token; its four waves take the QH + KH heads in turn and keep the
 // rotated head in LDS as fp32 between the two passes.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void rope_norm_store_kernel(
-    const T* __restrict__ proj, long stride, int QH, int KH, int D, int VW, const float* __restrict__ freqs,
+    const T* __restrict__ proj, long stride, int QH, int KH, int D, int VW, const double* __restrict__ freqs,
     int nrot, int layout, int unit, float eps, T* __restrict__ q_out, T* __restrict__ pool,
     const int* __restrict__ tok_pos, const long* __restrict__ tok_row) {
   extern __shared__ float heads_lds[];           // [4][D]
   const long t = blockIdx.x;
   const T* x = proj + t * stride;
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-  const float pos = (float)tok_pos[t];
+  const double pos = (double)tok_pos[t];
   T* row = pool + tok_row[t] * (long)(KH * D + VW);
   float* buf = heads_lds + wave * D;
   for (int u0 = 0; u0 < QH + KH; u0 += 256 / WAVE) {          // the same trip count for every wave
@@ -32,7 +32,10 @@ __global__ __launch_bounds__(256) void rope_norm_store_kernel(
         const int ia = layout == 0 ? 2 * i : i, ib = layout == 0 ? 2 * i + 1 : i + nrot;
         const float a = ldf(src + ia), b = ldf(src + ib);
         float sn, cs;
-        sincosf(pos * freqs[i], &sn, &cs);
+        // the angle in float64, reduced to [-pi, pi] before it is rounded: far positions keep their precision
+        double turns = pos * freqs[i] * 0.15915494309189535;      // angle / 2 pi
+        turns -= rint(turns);
+        sincosf((float)(turns * 6.283185307179586), &sn, &cs);
         const float ra = a * cs - b * sn, rb = b * cs + a * sn;
         buf[ia] = ra;
         buf[ib] = rb;
@@ -68,7 +71,8 @@ torch::Tensor rope_norm_store(torch::Tensor proj, int64_t QH, int64_t KH, int64_
   TORCH_CHECK(tok_row.numel() == T_ && tok_pos.numel() == T_);
   TORCH_CHECK(layout == 0 || layout == 1, "layout: 0 neighbouring pairs, 1 halves");
   const int nrot = freqs.numel();
-  if (nrot > 0) check_f32(freqs, "freqs");
+  if (nrot > 0)
+    TORCH_CHECK(freqs.is_cuda() && freqs.scalar_type() == at::kDouble && freqs.is_contiguous(), "freqs: float64 device tensor");
   TORCH_CHECK(2 * nrot <= D, "rotated entries lie inside a head");
   TORCH_CHECK(pool.is_contiguous() && pool.dim() == 2 && pool.size(1) == KH * D + VW &&
               pool.scalar_type() == proj.scalar_type());
@@ -78,7 +82,7 @@ torch::Tensor rope_norm_store(torch::Tensor proj, int64_t QH, int64_t KH, int64_
   auto stream = at::cuda::getCurrentHIPStream();
   RAGGED_DISPATCH(proj, hipLaunchKernelGGL((rope_norm_store_kernel<T>), dim3(T_), dim3(256),
       (size_t)4 * D * sizeof(float), stream, (const T*)proj.data_ptr(), (long)proj.stride(0), (int)QH, (int)KH,
-      (int)D, (int)VW, nrot > 0 ? freqs.data_ptr<float>() : nullptr, nrot, (int)layout, unit ? 1 : 0, (float)eps,
+      (int)D, (int)VW, nrot > 0 ? freqs.data_ptr<double>() : nullptr, nrot, (int)layout, unit ? 1 : 0, (float)eps,
       (T*)q.data_ptr(), (T*)pool.data_ptr(), tok_pos.data_ptr<int>(), tok_row.data_ptr<long>()));
   return q;
 }

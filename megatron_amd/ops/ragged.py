@@ -516,19 +516,33 @@ def _map_mfma_ok(q, dim, vdim) -> bool:
             and os.environ.get("MEGATRON_AMD_NO_MFMA_MAPS", "0") != "1")
 
 
-def _map_split(batch, nblk):
-    return max(1, min((batch.max_context + 63) // 64, 1024 // max(nblk, 1), 64))
+def _map_split(batch, nblk, vdim):
+    """Key splits of the matrix-core kernel for steps with few row tiles.  Every split writes fp32
+    partial results of vdim columns a row, so few long splits beat many short ones: measured best
+    (4 and 16 requests at 2048 positions) at about 512 workgroups for values up to 128 wide and 256
+    for wider ones (MEGATRON_AMD_MAP_SPLIT_WGS overrides)."""
+    wgs = int(os.environ.get("MEGATRON_AMD_MAP_SPLIT_WGS", "512" if vdim <= 128 else "256"))
+    return max(1, min((batch.max_context + 63) // 64, wgs // max(nblk, 1), 64))
+
+
+def _map_tiles(batch, rep, key_heads, device):
+    """Work list of the matrix-core kernel -> (tiles, rows a tile).  64 rows a workgroup (one row
+    tile a wave); MEGATRON_AMD_MAP_TILE_ROWS=128 selects two row tiles a wave, which measured
+    slower on whole prompts (more registers, fewer waves a SIMD) and is kept for experiments."""
+    rows = int(os.environ.get("MEGATRON_AMD_MAP_TILE_ROWS", "64"))
+    return batch.row_tiles(rep, device, rows), rows
 
 
 def map_attention(q, pool, heads, kv_heads, maps, dim, vdim, scale, softcap, batch):
     """-> fp32 [T, heads * maps * vdim]: the result of every softmax map of every head"""
     if _native_g(q):
         if _map_mfma_ok(q, dim, vdim):
-            tiles = batch.row_tiles(heads // kv_heads, q.device)
-            nsplit = _map_split(batch, tiles.shape[0] * kv_heads * maps)
+            tiles, rows = _map_tiles(batch, heads // kv_heads, kv_heads * maps, q.device)
+            nsplit = _map_split(batch, tiles.shape[0] * kv_heads * maps, vdim)
             return _G.map_attention_mfma(q, _none(q.device), pool, int(heads), int(kv_heads), int(maps), int(dim),
                                          int(vdim), float(scale), float(softcap), tiles, batch.cu_tokens,
-                                         batch.start_pos, batch.block_tables, int(batch.block_size), int(nsplit))
+                                         batch.start_pos, batch.block_tables, int(batch.block_size), int(nsplit),
+                                         rows)
         return _G.map_attention(q, pool, int(heads), int(kv_heads), int(maps), int(dim), int(vdim), float(scale),
                                 float(softcap), batch.tok_req, batch.tok_pos, batch.block_tables,
                                 int(batch.block_size))
@@ -541,11 +555,11 @@ def softcap_gated_attention(q, gate, pool, heads, kv_heads, dim, vdim, scale, so
     if _native_g(q):
         if _map_mfma_ok(q, dim, vdim):
             # matrix-core kernel, gate applied when the result leaves the accumulators
-            tiles = batch.row_tiles(heads // kv_heads, q.device)
-            nsplit = _map_split(batch, tiles.shape[0] * kv_heads)
+            tiles, rows = _map_tiles(batch, heads // kv_heads, kv_heads, q.device)
+            nsplit = _map_split(batch, tiles.shape[0] * kv_heads, vdim)
             return _G.map_attention_mfma(q, gate, pool, int(heads), int(kv_heads), 1, int(dim), int(vdim),
                                          float(scale), float(softcap), tiles, batch.cu_tokens, batch.start_pos,
-                                         batch.block_tables, int(batch.block_size), int(nsplit))
+                                         batch.block_tables, int(batch.block_size), int(nsplit), rows)
         A = map_attention(q, pool, heads, kv_heads, 1, dim, vdim, scale, softcap, batch)
         return _G.gate_finish(A, gate, q.dtype == torch.bfloat16)
     A = ref.map_attention(q, pool, heads, kv_heads, 1, dim, vdim, scale, softcap, batch)

@@ -591,7 +591,8 @@ def scaled_freqs(dims, base, scaling=None, device=None):
     low, high, original): a wavelength 2 pi / f below original/high keeps f, one
     above original/low uses f / factor, and between them
     s = (original / wavelength - low) / (high - low) blends (1 - s) f / factor + s f.
-    Rounded once to fp32."""
+    Kept in float64: at position p the angle p f_i is formed in float64 and reduced to
+    (-pi, pi] before it is rounded to fp32, so far positions lose no precision."""
     i = torch.arange(dims // 2, dtype=torch.float64)
     f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims)
     if scaling:
@@ -601,7 +602,7 @@ def scaled_freqs(dims, base, scaling=None, device=None):
         s = (orig / wl - low) / (high - low)
         mid = (1.0 - s) * f / factor + s * f
         f = torch.where(wl < orig / high, f, torch.where(wl > orig / low, f / factor, mid))
-    return f.to(torch.float32).to(device)
+    return f.to(device)
 
 
 ROT_LAYOUTS = {"pairs": 0, "halves": 1}
@@ -613,14 +614,18 @@ def _rotate_layout(x, pos, freqs, layout):
     n = freqs.numel()
     if n == 0:
         return x
-    if layout == "pairs":
-        return _rotate_pairs(x, pos, freqs)
-    ang = pos.float()[:, None, None] * freqs.float()[None, None, :]
+    ang = torch.remainder(pos.double()[:, None, None] * freqs.double()[None, None, :] + math.pi, 2.0 * math.pi) - math.pi
+    ang = ang.float()
     c, s = torch.cos(ang), torch.sin(ang)
-    u, v = x[..., :n], x[..., n:2 * n]
     out = x.clone()
-    out[..., :n] = u * c - v * s
-    out[..., n:2 * n] = v * c + u * s
+    if layout == "pairs":
+        u, v = x[..., 0:2 * n:2], x[..., 1:2 * n:2]
+        out[..., 0:2 * n:2] = u * c - v * s
+        out[..., 1:2 * n:2] = v * c + u * s
+    else:
+        u, v = x[..., :n], x[..., n:2 * n]
+        out[..., :n] = u * c - v * s
+        out[..., n:2 * n] = v * c + u * s
     return out
 
 
