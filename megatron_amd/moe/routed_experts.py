@@ -110,13 +110,20 @@ class RoutedExpertsMLP(nn.Module):
         inv[order] = torch.arange(order.numel(), device=order.device)
         xs = h.index_select(0, torch.div(order, K, rounding_mode="floor"))
         w_first = self.w_gate_up if self.gated else self.w_up
-        if self._grouped_ok(h):
+        down = None
+        if self._grouped_ok(h) and not getattr(self, "_grouped_refused", False):
             # one grouped GEMM per linear over the sorted pairs, group ends on the device: no host read
             offs = torch.cumsum(torch.bincount(flat, minlength=E), 0).to(torch.int32)
-            gu = torch._grouped_mm(xs, w_first.transpose(1, 2), offs=offs)
-            down = torch._grouped_mm(self._glu(gu, self.limit, h.dtype),
-                                     self.w_down.transpose(1, 2), offs=offs)
-        else:
+            try:
+                gu = torch._grouped_mm(xs, w_first.transpose(1, 2), offs=offs)
+                down = torch._grouped_mm(self._glu(gu, self.limit, h.dtype),
+                                         self.w_down.transpose(1, 2), offs=offs)
+            except RuntimeError as e:          # a shape the vendor's grouped GEMM does not take
+                import warnings
+
+                warnings.warn(f"grouped GEMM refused these expert sizes ({e}); one GEMM per expert instead")
+                self._grouped_refused = True
+        if down is None:
             counts = torch.bincount(flat, minlength=E).tolist()   # the step's host read
             down = torch.empty(T * K, h.shape[1], dtype=h.dtype, device=h.device)
             at = 0
