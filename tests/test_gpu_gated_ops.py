@@ -85,23 +85,23 @@ SHAPES = [(4, 2, 1, 24, 24), (3, 3, 2, 80, 40), (6, 1, 1, 144, 144), (2, 2, 2, 1
           (2, 2, 2, 160, 128), (16, 8, 1, 128, 128), (4, 1, 2, 128, 256)]
 
 
-@pytest.fixture(params=[64, 128], ids=["rows64", "rows128"])
-def tile_rows(request, monkeypatch):
-    """both tile sizes of the matrix-core kernel, whatever the step's size would choose"""
-    monkeypatch.setenv("MEGATRON_AMD_MAP_TILE_ROWS", str(request.param))
-    return request.param
+@pytest.fixture(params=[(torch.float32, 64), (torch.bfloat16, 64), (torch.bfloat16, 128)],
+                ids=["float32", "bfloat16-rows64", "bfloat16-rows128"])
+def dtype_tiles(request, monkeypatch):
+    """fp32 (VALU kernel) and bf16 with both tile sizes of the matrix-core kernel, whatever the step's
+    size would choose; -> the storage dtype"""
+    monkeypatch.setenv("MEGATRON_AMD_MAP_TILE_ROWS", str(request.param[1]))
+    return request.param[0]
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape", SHAPES + [(6, 3, 1, 40, 72), (2, 2, 2, 200, 136)])
 @pytest.mark.parametrize("starts", [STARTS, LONG], ids=["short", "long"])
 @pytest.mark.parametrize("cap", [0.0, 3.0])
-def test_map_attention(dtype, shape, starts, cap, tile_rows):
+def test_map_attention(dtype_tiles, shape, starts, cap):
     """heads, kv heads, maps, dim, vdim; page 16; long contexts beside short ones make the bf16 kernel
     split the key tiles; the shapes cover every matrix-core instantiation and sizes it does not take"""
-    if dtype == torch.float32 and tile_rows == 128:
-        pytest.skip("fp32 runs on the VALU kernel: no tiles")
     R = _need()
+    dtype = dtype_tiles
     H, G, M, D, V = shape
 
     def run(dev, dt):
@@ -115,14 +115,12 @@ def test_map_attention(dtype, shape, starts, cap, tile_rows):
     _close(g, c, dtype, "attention")
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape", [s for s in SHAPES if s[2] == 1])
 @pytest.mark.parametrize("starts", [STARTS, LONG], ids=["short", "long"])
-def test_softcap_gated_attention(dtype, shape, starts, tile_rows):
+def test_softcap_gated_attention(dtype_tiles, shape, starts):
     """the gate is a strided view behind other columns, as a fused projection's slice is"""
-    if dtype == torch.float32 and tile_rows == 128:
-        pytest.skip("fp32 runs on the VALU kernel: no tiles")
     R = _need()
+    dtype = dtype_tiles
     H, G, _, D, V = shape
 
     def run(dev, dt):
@@ -159,13 +157,11 @@ def test_differential_attention(dtype, shape, starts):
     _close(g, c, dtype, "differential attention")
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_map_attention_prompt_tiles(dtype, tile_rows):
+def test_map_attention_prompt_tiles(dtype_tiles):
     """long portions: several row tiles per request; rows of one tile end in different key tiles; a last
     tile whose later row tiles are empty; a first row tile that ends before the key tile the second needs"""
-    if dtype == torch.float32 and tile_rows == 128:
-        pytest.skip("fp32 runs on the VALU kernel: no tiles")
     R = _need()
+    dtype = dtype_tiles
     H, G, M, D, V = 4, 2, 2, 64, 32
 
     def run(dev, dt):
